@@ -487,6 +487,54 @@ int tgis_delta_scan(const float* conv, int64_t C, const void* a, int64_t ld_a, c
                     const int32_t* positions, void* out, int64_t ld_out, int64_t B, int H, int G, int dk, int dv, int taps,
                     float eps, float unit_eps, float q_scale, int dtype, void* stream);
 
+/* ---- parallel-layer decoders with gated residuals (Mananex): windowed attention with a sink, rotation in the "rows" page
+ *      layout, a gated linear recurrence, the parallel residual update with a mix over depth.  T as above. */
+
+/* Interleaved-pair rotation of q (in place) and k (into its page slot), and the value write, of a step.  proj [T, ld] holds q
+ * at columns q_col0 + h dk, k at k_col0 + g dk, v at v_col0 + g dv.  Pair (2i, 2i + 1) of the first rot_dims channels of every
+ * q and k head turns by positions[t] * inv_freq[i] (angle, sine and cosine in fp32); the other channels pass. */
+int tgis_rope_rows_kv_write(void* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t v_col0, const float* inv_freq,
+                            const int32_t* positions, const int32_t* slots, void* k_pool, void* v_pool, int64_t T, int H, int G,
+                            int dk, int dv, int rot_dims, int dtype, void* stream);
+/* tgis_attn_varlen with a sliding window that keeps the first positions (window > 0: position i sees j <= i only if
+ * i - j < window or j < keep_first; kept keys stay at their positions; pages between them and the window are not read), a sink
+ * logit per query head in the softmax denominator (sink [H] fp32 or NULL: exp(sink[h]) is added once, unscaled, with no value),
+ * a sigmoid output gate (gate_per_head != 0: gate [T, >= H], one logit per (token, head); else gate [T, >= H dv]) and a constant
+ * factor out_scale on the output.  out may be a column range of a wider buffer (ld_out).  workspace as in tgis_attn_varlen_ext. */
+int tgis_attn_varlen_win(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
+                         int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B, void* out,
+                         int64_t ld_out, int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv,
+                         float scale, int window, int keep_first, const float* sink, const void* gate, int64_t ld_gate,
+                         int gate_per_head, float out_scale, void* workspace, int64_t workspace_bytes, int impl, int dtype,
+                         void* stream);
+/* Gated linear recurrence per (sequence, head), tokens in order, on columns of proj [T, ld]:
+ *   q = proj[q_col0 + h dk ..] (q_act 1: silu of it);  f = lower + (1 - lower) sigmoid(proj[f_col0 + h dk ..] + f_bias)  (fp32;
+ *   lower, f_bias [H dk] fp32 or NULL = 0);  v = proj[v_col0 + h dv ..];
+ *   S <- diag(f) S + (1 - f) v^T;  o = S^T q (the new state);  out = o / sqrt(mean(o^2) + eps) * gain[dv] * out_scale.
+ * state [slots][H][dk][dv] fp32 is read (zeros when the step starts at position 0) and written back.  dk, dv <= 256. */
+int tgis_gated_linear_scan(const void* proj, int64_t ld, int64_t q_col0, int64_t f_col0, int64_t v_col0, const float* f_bias,
+                           const float* lower, const float* gain, float* state, const int32_t* state_slots,
+                           const int32_t* cu_seqlens_q, const int32_t* positions, void* out, int64_t ld_out, float out_scale,
+                           int64_t B, int H, int dk, int dv, float eps, int q_act, int dtype, void* stream);
+/* tgis_moe_route with a bias on the router logits (router_b [E] fp32 or NULL) and, with softmax_top != 0, weights that are the
+ * softmax over the chosen logits only (0: the sigmoid of each chosen logit). */
+int tgis_moe_route_ext(const void* h, int64_t ld_h, const float* router_w, const float* router_b, const float* shared_gate_w,
+                       int softmax_top, int32_t* idx, float* weight, float* shared_gate, int64_t T, int64_t W, int E, int k,
+                       int dtype, void* stream);
+/* The residual update of a parallel layer (mixer a and feed-forward b read the same normed input) with gated residuals and a
+ * learned mix over depth, and the next norm, in one launch:
+ *   v = x + sigmoid(gate_a + gate_bias_a) (a + bias_a) + sigmoid(gate_b + gate_bias_b) (b + bias_b)
+ *   hist[n_prev] = v;  x_out = sum_{j <= n_prev} mix[j] hist[j]  (hist NULL: x_out = v);
+ *   y = x_out / sqrt(mean(x_out^2) + eps) * (pre_w + pre_add)  (pre_w NULL: none)
+ * a / b: [rows, ld] of `dtype`, or with slabs_x > 0 the fp32 split-K slabs of tgis_dense_gemm_partial (ld_x = their row
+ * stride); b, the biases [E], gate logits [rows, ld_gate] and gate biases [E] (all of `dtype`) may be NULL.
+ * hist: n_prev + 1 entries [rows, E] fp32, hist_stride floats apart; mix [n_prev + 1] fp32.  x_out may alias x. */
+int tgis_parallel_residual_f32(const float* x, const void* a, int64_t ld_a, int slabs_a, const void* bias_a, const void* gate_a,
+                               int64_t ld_gate_a, const void* gate_bias_a, const void* b, int64_t ld_b, int slabs_b,
+                               const void* bias_b, const void* gate_b, int64_t ld_gate_b, const void* gate_bias_b, int dtype,
+                               float* hist, int n_prev, int64_t hist_stride, const float* mix, float* x_out, const float* pre_w,
+                               float pre_add, void* y, int y_dtype, int64_t rows, int64_t E, float eps, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -35,9 +35,43 @@ struct AttnExt {
     int key_splits;
     float* partial;
     int64_t partial_tokens;  // tokens of the step (the partial results' second extent)
+    //   window > 0: a query at position i sees key j <= i only if i - j < window or j < keep_first (a sliding window that
+    //               also keeps the first positions of the sequence, at their true positions); not combined with chunk
+    //   sink:       per query head, exp(sink[h]) joins the softmax denominator: a slot without key or value, not scaled
+    //   gate_per_head: the gate holds ONE number per (token, head), gate[t][h], instead of one per output channel
+    //   out_scale:  the output is multiplied by this where it is written
+    int window = 0;
+    int keep_first = 0;
+    const float* sink = nullptr;
+    int gate_per_head = 0;
+    float out_scale = 1.f;
 };
 __device__ __forceinline__ float sigmoid_f32(float z) { return 1.f / (1.f + expf(-z)); }
-__device__ __forceinline__ int first_visible(const AttnExt& e, int pos) { return e.chunk > 0 && pos > 0 ? pos / e.chunk * e.chunk : 0; }
+__device__ __forceinline__ int first_visible(const AttnExt& e, int pos) {
+    if (e.window > 0) return max(pos - e.window + 1, 0);
+    return e.chunk > 0 && pos > 0 ? pos / e.chunk * e.chunk : 0;
+}
+// key j of a query at position pos whose window / block starts at lo
+__device__ __forceinline__ bool key_visible(const AttnExt& e, int key, int pos, int lo) { return key <= pos && (key >= lo || key < e.keep_first); }
+// The pages (or 64-key chunks) a walk visits: the first `nkeep` units hold kept first positions, then it continues at unit `u0`.
+__device__ __forceinline__ int kept_units(const AttnExt& e, int u0, int unit) { return min((e.keep_first + unit - 1) / unit, u0); }
+__device__ __forceinline__ int walk_unit(int i, int nkeep, int u0) { return i < nkeep ? i : u0 + (i - nkeep); }
+// Softmax statistics (m, l) of a finished column take the sink in: returns the factor for the unnormalised sums, l becomes the
+// full denominator.  m is finite (a query always sees its own key).
+__device__ __forceinline__ float fold_sink(const AttnExt& e, int head, float m, float& l) {
+    if (!e.sink) return 1.f;
+    const float sk = e.sink[head];
+    const float mm = fmaxf(m, sk);
+    const float f = expf(m - mm);
+    l = l * f + expf(sk - mm);
+    return f;
+}
+// what multiplies head `head` of token t where it is written (the per-head gate and the output scale)
+template <typename T> __device__ __forceinline__ float head_out_factor(const AttnExt& e, int64_t t, int head) {
+    float f = e.out_scale;
+    if (e.gate && e.gate_per_head) f *= sigmoid_f32((float)reinterpret_cast<const T*>(e.gate)[t * e.ld_gate + head]);
+    return f;
+}
 
 template <typename T> __device__ __forceinline__ float ldf(const T* p) { return (float)*p; }
 
@@ -246,17 +280,19 @@ __global__ __launch_bounds__(1024) void attn_varlen_kernel(
     float o[DV_PER_LANE];
 #pragma unroll
     for (int c = 0; c < DV_PER_LANE; ++c) o[c] = 0.f;
-    for (int base = lo / 64 * 64 + sp * 64; base < nkeys; base += S * 64) {
+    const int c0 = lo / 64, nkc = kept_units(ext, c0, 64), nchunks = nkc + (nkeys + 63) / 64 - c0;
+    for (int ci = sp; ci < nchunks; ci += S) {
+        const int base = walk_unit(ci, nkc, c0) * 64;
         const int j = base + lane;
         float s = -INFINITY;
-        if (j < nkeys && j >= lo) {
+        if (key_visible(ext, j, pos, lo)) {
             const int64_t page = table[j / PAGE];
             s = dot_row<T>(myq, k_pool + ((page * G + g) * PAGE + (j % PAGE)) * dk, dk);
             if (ext.r1) s -= r1h * log1pf(r2h * (float)(pos - j));
         }
         const float mn = fmaxf(m, wave_max(s));  // finite: key `base` is visible
         const float corr = expf(m - mn);         // exp(-inf) = 0 on the first chunk
-        const float p = (j < nkeys && j >= lo) ? expf(s - mn) : 0.f;
+        const float p = key_visible(ext, j, pos, lo) ? expf(s - mn) : 0.f;
         l = l * corr + wave_sum(p);
         m = mn;
 #pragma unroll
@@ -264,7 +300,7 @@ __global__ __launch_bounds__(1024) void attn_varlen_kernel(
         for (int half = 0; half < 64 / PAGE; ++half) {
             const int first = base + half * PAGE;
             if (first >= nkeys) break;
-            if (first + PAGE <= lo) continue;  // a page before the query's block: all its weights are zero
+            if (first + PAGE <= lo && first >= ext.keep_first) continue;  // a page before the query's block: all its weights are zero
             const int n = min(PAGE, nkeys - first);
             const int64_t page = table[first / PAGE];
 #pragma unroll
@@ -312,12 +348,14 @@ __global__ __launch_bounds__(1024) void attn_varlen_kernel(
                 if (lane + 64 * c < dv) acc[c] += other[2 + lane + 64 * c] * w;
         }
         l = ll;
+        m = mm;
 #pragma unroll
         for (int c = 0; c < DV_PER_LANE; ++c) o[c] = acc[c];
     }
-    const float inv = 1.f / l;
+    const float sink_f = fold_sink(ext, g * Rall + r0 + r, m, l);
+    const float inv = sink_f / l * head_out_factor<T>(ext, t, g * Rall + r0 + r);
     T* orow = out + (int64_t)t * ld_out + (int64_t)(g * Rall + r0 + r) * dv;
-    const T* grow = ext.gate ? reinterpret_cast<const T*>(ext.gate) + (int64_t)t * ext.ld_gate + (int64_t)(g * Rall + r0 + r) * dv : nullptr;
+    const T* grow = (ext.gate && !ext.gate_per_head) ? reinterpret_cast<const T*>(ext.gate) + (int64_t)t * ext.ld_gate + (int64_t)(g * Rall + r0 + r) * dv : nullptr;
 #pragma unroll
     for (int c = 0; c < DV_PER_LANE; ++c)
         if (lane + 64 * c < dv) orow[lane + 64 * c] = (T)(o[c] * inv * (grow ? sigmoid_f32(ldf(grow + lane + 64 * c)) : 1.f));
@@ -360,6 +398,8 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
     // blocks: positions grow with the columns, so the tile's first column has the earliest first visible key
     const int lo = first_visible(ext, pos);
     const int page0 = first_visible(ext, ctx - qlen + tile * 32 / R) / PAGE;
+    // the walk: pages with kept first positions that lie before the window, then the window's pages
+    const int nkeep = kept_units(ext, page0, PAGE), nvis = nkeep + npages - page0;
     const float r1h = ext.r1 ? ext.r1[g * R + r] : 0.f, r2h = ext.r1 ? ext.r2[g * R + r] : 0.f;
     // Q^T fragments: lane (column c, half h) holds 8 consecutive channels of its column's query per 16-channel step
     V8 qf[DK16];
@@ -376,21 +416,22 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
     // the K fragments of a page are asked for one page ahead: a page costs its arithmetic, not a round trip to memory
     V8 kf[DK16];
     int64_t page = 0;
-    const int pstart = page0 + (split ? (int)blockIdx.x * nw + wave : 0);
-    if (pstart < npages) {
-        page = table[pstart];
+    const int pstart = split ? (int)blockIdx.x * nw + wave : 0;
+    if (pstart < nvis) {
+        page = table[walk_unit(pstart, nkeep, page0)];
         const T* kp = k_pool + ((page * G + g) * PAGE + c) * dk + h * 8;
 #pragma unroll
         for (int s = 0; s < DK16; ++s) kf[s] = s < nks ? *reinterpret_cast<const V8*>(kp + s * 16) : V8{};
     }
-    for (int p = pstart; p < npages; p += pstep) {
+    for (int pi = pstart; pi < nvis; pi += pstep) {
+        const int p = walk_unit(pi, nkeep, page0);
         f32x16 S = {};
 #pragma unroll
         for (int s = 0; s < DK16; ++s)
             if (s < nks) S = mfma32(kf[s], qf[s], S);
         const int64_t this_page = page;
-        if (p + pstep < npages) {
-            page = table[p + pstep];
+        if (pi + pstep < nvis) {
+            page = table[walk_unit(pi + pstep, nkeep, page0)];
             const T* kp = k_pool + ((page * G + g) * PAGE + c) * dk + h * 8;
 #pragma unroll
             for (int s = 0; s < DK16; ++s) kf[s] = s < nks ? *reinterpret_cast<const V8*>(kp + s * 16) : V8{};
@@ -413,14 +454,14 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int key = base + (i >> 2) * 8 + (i & 3);
-                S[i] = (key <= pos && key >= lo) ? S[i] * scale - r1h * __logf(1.f + r2h * (float)(pos - key)) : -INFINITY;
+                S[i] = key_visible(ext, key, pos, lo) ? S[i] * scale - r1h * __logf(1.f + r2h * (float)(pos - key)) : -INFINITY;
                 mx = fmaxf(mx, S[i]);
             }
         } else {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int key = base + (i >> 2) * 8 + (i & 3);
-                S[i] = (key <= pos && key >= lo) ? S[i] * scale : -INFINITY;
+                S[i] = key_visible(ext, key, pos, lo) ? S[i] * scale : -INFINITY;
                 mx = fmaxf(mx, S[i]);
             }
         }
@@ -509,9 +550,10 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
             }
             return;
         }
-        const float inv = 1.f / ll;
+        const float sink_f = fold_sink(ext, g * R + r, mm, ll);
+        const float inv = sink_f / ll * head_out_factor<T>(ext, t0 + tq, g * R + r);
         T* orow = out + (int64_t)(t0 + tq) * ld_out + (int64_t)(g * R + r) * dv + h * 4;
-        const T* grow = ext.gate ? reinterpret_cast<const T*>(ext.gate) + (int64_t)(t0 + tq) * ext.ld_gate + (int64_t)(g * R + r) * dv + h * 4 : nullptr;
+        const T* grow = (ext.gate && !ext.gate_per_head) ? reinterpret_cast<const T*>(ext.gate) + (int64_t)(t0 + tq) * ext.ld_gate + (int64_t)(g * R + r) * dv + h * 4 : nullptr;
         for (int grp = wave; grp < nvt * 4; grp += nw) {
             const int t = grp >> 2, j = grp & 3;
             float acc[4] = {0.f, 0.f, 0.f, 0.f};
@@ -530,9 +572,10 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
         return;
     }
     if (!live) return;
-    const float inv = 1.f / lsum;
+    const float sink_f = fold_sink(ext, g * R + r, m, lsum);
+    const float inv = sink_f / lsum * head_out_factor<T>(ext, t0 + tq, g * R + r);
     T* orow = out + (int64_t)(t0 + tq) * ld_out + (int64_t)(g * R + r) * dv + h * 4;
-    const T* grow = ext.gate ? reinterpret_cast<const T*>(ext.gate) + (int64_t)(t0 + tq) * ext.ld_gate + (int64_t)(g * R + r) * dv + h * 4 : nullptr;
+    const T* grow = (ext.gate && !ext.gate_per_head) ? reinterpret_cast<const T*>(ext.gate) + (int64_t)(t0 + tq) * ext.ld_gate + (int64_t)(g * R + r) * dv + h * 4 : nullptr;
 #pragma unroll
     for (int t = 0; t < DVT; ++t)
         if (t < nvt) {
@@ -561,10 +604,11 @@ __global__ __launch_bounds__(64) void attn_combine_splits_kernel(const float* __
     const float ol = lane < X ? p0[lane * stride + 1] : 0.f;
     const float mm = wave_max(om);
     const float e = om == -INFINITY ? 0.f : expf(om - mm);
-    const float ll = wave_sum(ol * e);
-    wx[lane] = e / ll;
+    float ll = wave_sum(ol * e);
+    const float sink_f = fold_sink(ext, head, mm, ll);
+    wx[lane] = e * sink_f / ll * head_out_factor<T>(ext, t, head);
     __syncthreads();
-    const T* grow = ext.gate ? reinterpret_cast<const T*>(ext.gate) + t * ext.ld_gate + (int64_t)head * dv : nullptr;
+    const T* grow = (ext.gate && !ext.gate_per_head) ? reinterpret_cast<const T*>(ext.gate) + t * ext.ld_gate + (int64_t)head * dv : nullptr;
     for (int c = lane; c < dv; c += 64) {
         float acc = 0.f;
         for (int x = 0; x < X; ++x) acc += p0[x * stride + 2 + c] * wx[x];
@@ -611,6 +655,8 @@ __global__ __launch_bounds__(256) void attn_varlen_staged_kernel(
     const int lo = first_visible(ext, pos);
     const int wg_page0 = first_visible(ext, ctx - qlen + (int)blockIdx.x * 128 / R) / PAGE;
     const int my_page0 = tile_live ? first_visible(ext, ctx - qlen + tile * 32 / R) / PAGE : 0;
+    // the workgroup's walk: pages with kept first positions that lie before its window pages, then those
+    const int wg_nkeep = kept_units(ext, wg_page0, PAGE), wg_nvis = wg_nkeep + wg_pages - wg_page0;
     const float r1h = ext.r1 ? ext.r1[g * R + r] : 0.f, r2h = ext.r1 ? ext.r2[g * R + r] : 0.f;
     V8 qf[DK16];
     const T* qrow = q + (int64_t)(t0 + tq) * ldq + (int64_t)(g * R + r) * dk + h * 8;
@@ -638,8 +684,9 @@ __global__ __launch_bounds__(256) void attn_varlen_staged_kernel(
             vreg[i] = e < velems ? *reinterpret_cast<const V8*>(vp + e) : V8{};
         }
     };
-    fetch(wg_page0);
-    for (int p = wg_page0; p < wg_pages; ++p) {
+    fetch(walk_unit(0, wg_nkeep, wg_page0));
+    for (int pi = 0; pi < wg_nvis; ++pi) {
+        const int p = walk_unit(pi, wg_nkeep, wg_page0);
         __syncthreads();  // the page before is consumed
 #pragma unroll
         for (int i = 0; i < KL; ++i) {
@@ -662,8 +709,8 @@ __global__ __launch_bounds__(256) void attn_varlen_staged_kernel(
             }
         }
         __syncthreads();
-        if (p + 1 < wg_pages) fetch(p + 1);
-        if (p >= my_pages || p < my_page0) continue;
+        if (pi + 1 < wg_nvis) fetch(walk_unit(pi + 1, wg_nkeep, wg_page0));
+        if (p >= my_pages || (p < my_page0 && p * PAGE >= ext.keep_first)) continue;
         f32x16 S = {};
 #pragma unroll
         for (int s = 0; s < DK16; ++s)
@@ -674,14 +721,14 @@ __global__ __launch_bounds__(256) void attn_varlen_staged_kernel(
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int key = base + (i >> 2) * 8 + (i & 3);
-                S[i] = (key <= pos && key >= lo) ? S[i] * scale - r1h * __logf(1.f + r2h * (float)(pos - key)) : -INFINITY;
+                S[i] = key_visible(ext, key, pos, lo) ? S[i] * scale - r1h * __logf(1.f + r2h * (float)(pos - key)) : -INFINITY;
                 mx = fmaxf(mx, S[i]);
             }
         } else {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int key = base + (i >> 2) * 8 + (i & 3);
-                S[i] = (key <= pos && key >= lo) ? S[i] * scale : -INFINITY;
+                S[i] = key_visible(ext, key, pos, lo) ? S[i] * scale : -INFINITY;
                 mx = fmaxf(mx, S[i]);
             }
         }
@@ -727,9 +774,10 @@ __global__ __launch_bounds__(256) void attn_varlen_staged_kernel(
     }
     lsum += __shfl_xor(lsum, 32, 64);
     if (!live) return;
-    const float inv = 1.f / lsum;
+    const float sink_f = fold_sink(ext, g * R + r, m, lsum);
+    const float inv = sink_f / lsum * head_out_factor<T>(ext, t0 + tq, g * R + r);
     T* orow = out + (int64_t)(t0 + tq) * ld_out + (int64_t)(g * R + r) * dv + h * 4;
-    const T* grow = ext.gate ? reinterpret_cast<const T*>(ext.gate) + (int64_t)(t0 + tq) * ext.ld_gate + (int64_t)(g * R + r) * dv + h * 4 : nullptr;
+    const T* grow = (ext.gate && !ext.gate_per_head) ? reinterpret_cast<const T*>(ext.gate) + (int64_t)(t0 + tq) * ext.ld_gate + (int64_t)(g * R + r) * dv + h * 4 : nullptr;
 #pragma unroll
     for (int t = 0; t < DVT; ++t)
         if (t < nvt) {
@@ -858,12 +906,66 @@ __global__ __launch_bounds__(256) void latent_kv_write_kernel(const T* __restric
     if ((dr & 1) && lane == 0) dst[dr - 1] = qr[dr - 1];
 }
 
+// Rotation and cache write of designs that rotate q and k: pair (2i, 2i + 1) of the first `rdims` channels of every q and k
+// head turns by position * inv_freq[i] (angle and sin / cos in fp32), the rest pass.  q is rotated in place, k goes to its
+// page slot rotated, v to its slot as projected (v_inline) or stays for the transposing writer.
+// grid (token, ceil((H + G) / 4) [+ value blocks]): a wave per q / k head.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_rows_kv_write_kernel(T* __restrict__ qkv, int64_t ld, int64_t q_col0, int64_t k_col0,
+                                                                 int64_t v_col0, const float* __restrict__ inv_freq,
+                                                                 const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
+                                                                 T* __restrict__ k_pool, T* __restrict__ v_pool, int H, int G, int dk,
+                                                                 int dv, int rdims, int v_inline) {
+    const int64_t t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int slot = slots[t];
+    const int64_t page = slot / PAGE;
+    const int off = slot % PAGE;
+    T* row = qkv + t * ld;
+    const int head_blocks = (H + G + 3) / 4;
+    if ((int)blockIdx.y >= head_blocks) {
+        const T* vrow = row + v_col0;
+        const int i0 = ((int)blockIdx.y - head_blocks) * 1024;
+        const int i1 = min(i0 + 1024, G * dv);
+        for (int i = i0 + threadIdx.x; i < i1; i += blockDim.x) {
+            const int g = i / dv, c = i - g * dv;
+            v_pool[((page * G + g) * dv + c) * PAGE + off] = vrow[i];
+        }
+        return;
+    }
+    const int h = blockIdx.y * 4 + wave;
+    if (h >= H + G) return;
+    const bool is_q = h < H;
+    T* src = is_q ? row + q_col0 + (int64_t)h * dk : row + k_col0 + (int64_t)(h - H) * dk;
+    T* dst = is_q ? src : k_pool + ((page * G + (h - H)) * PAGE + off) * dk;
+    const float pos = (float)positions[t];
+    for (int i = lane; 2 * i < dk; i += 64) {
+        const int d = 2 * i;
+        if (d + 1 >= dk) {  // an odd width's last channel has no partner
+            dst[d] = src[d];
+            continue;
+        }
+        const float u = ldf(src + d), v = ldf(src + d + 1);
+        if (d + 1 < rdims) {
+            float sn, cs;
+            sincosf(pos * inv_freq[i], &sn, &cs);
+            dst[d] = (T)(u * cs - v * sn);
+            dst[d + 1] = (T)(v * cs + u * sn);
+        } else if (!is_q) {
+            dst[d] = src[d];
+            dst[d + 1] = src[d + 1];
+        }
+    }
+}
+
 template <typename T, int DK16, int DVT>
 void launch_mfma_one(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* bt, int64_t bt_ld,
                      const int32_t* ctx_lens, const int32_t* cu_q, int B, void* out, int64_t ld_out, int64_t max_q_len, int H, int G,
                      int dk, int dv, float scale, int64_t max_ctx, AttnExt ext, hipStream_t st) {
     const int R = H / G;
     const bool split = max_q_len * R <= 32;
+    // a windowed query walks its window's pages and the kept first ones, whatever the context
+    if (ext.window > 0) max_ctx = std::min<int64_t>(max_ctx, (int64_t)ext.window + ext.keep_first + 2 * PAGE);
     int nw = 4;
     size_t lds = 0;
     unsigned gx = 1;
@@ -1116,4 +1218,59 @@ extern "C" int tgis_latent_kv_write(const void* q, int64_t ldq, void* ckv, int64
                                                      (const float*)nullptr, (TT*)v_pool, T, 1, kv_rank));
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
+}
+
+// Interleaved-pair rotation of q (in place) and k (into its page slot) and the value write of a step, for the "rows" page
+// layout of tgis_attn_varlen.  proj [T, ld] holds q at columns q_col0 + h dk, k at k_col0 + g dk, v at v_col0 + g dv; pair
+// (2i, 2i + 1) of the first rot_dims channels of every head turns by positions[t] * inv_freq[i] (fp32 angle), the rest pass.
+extern "C" int tgis_rope_rows_kv_write(void* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t v_col0, const float* inv_freq,
+                                       const int32_t* positions, const int32_t* slots, void* k_pool, void* v_pool, int64_t T, int H,
+                                       int G, int dk, int dv, int rot_dims, int dtype, void* stream) {
+    TGIS_CHECK_ARG(proj && positions && slots && k_pool && v_pool && (inv_freq || rot_dims == 0), "tgis_rope_rows_kv_write: null tensor");
+    TGIS_CHECK_ARG(H >= 1 && G >= 1 && dk >= 1 && dv >= 1 && rot_dims >= 0 && rot_dims <= dk && rot_dims % 2 == 0 && q_col0 >= 0 &&
+                       k_col0 >= 0 && v_col0 >= 0 && ld >= q_col0 + (int64_t)H * dk && ld >= k_col0 + (int64_t)G * dk &&
+                       ld >= v_col0 + (int64_t)G * dv,
+                   "tgis_rope_rows_kv_write: bad geometry (H %d, G %d, dk %d, dv %d, rot_dims %d, ld %ld)", H, G, dk, dv, rot_dims, (long)ld);
+    TGIS_CHECK_ARG(dtype == TGIS_F16 || dtype == TGIS_BF16 || dtype == TGIS_F32, "tgis_rope_rows_kv_write: bad dtype");
+    if (T == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    TgisTimedScope timed(TGIS_OP_ROPE_KV, st);
+    const int v_inline = T < 512 ? 1 : 0;
+    const int v_blocks = v_inline ? (int)cdiv64((int64_t)G * dv, 1024) : 0;
+    TGIS_ATTN_BY_DTYPE(dtype, hipLaunchKernelGGL(rope_rows_kv_write_kernel<TT>, dim3((unsigned)T, (unsigned)((H + G + 3) / 4 + v_blocks)), dim3(256),
+                                                 0, st, (TT*)proj, ld, q_col0, k_col0, v_col0, inv_freq, positions, slots, (TT*)k_pool,
+                                                 (TT*)v_pool, H, G, dk, dv, rot_dims, v_inline));
+    if (!v_inline)
+        TGIS_ATTN_BY_DTYPE(dtype, hipLaunchKernelGGL(v_write_kernel<TT>, dim3((unsigned)cdiv64(T, 32), (unsigned)cdiv64((int64_t)G * dv, 64)),
+                                                     dim3(256), 0, st, (const TT*)proj, ld, v_col0, slots, (const TT*)nullptr, (int64_t)0,
+                                                     (const float*)nullptr, (TT*)v_pool, T, G, dv));
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+// tgis_attn_varlen with a sliding window that also keeps the first positions (window > 0: position i sees j <= i only if
+// i - j < window or j < keep_first; pages between the kept ones and the window are never touched), a sink logit per query head
+// in the softmax denominator (sink [H] fp32 or NULL), a sigmoid output gate (gate_per_head: one number per (token, head),
+// gate [T, >= H]; else one per channel, gate [T, >= H dv]) and a constant factor on the output.  out may be a column range of
+// a wider buffer (ld_out).  workspace: as for tgis_attn_varlen_ext.
+extern "C" int tgis_attn_varlen_win(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
+                                    int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B, void* out,
+                                    int64_t ld_out, int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv,
+                                    float scale, int window, int keep_first, const float* sink, const void* gate, int64_t ld_gate,
+                                    int gate_per_head, float out_scale, void* workspace, int64_t workspace_bytes, int impl, int dtype,
+                                    void* stream) {
+    TGIS_CHECK_ARG(window >= 0 && keep_first >= 0 && (window > 0 || keep_first == 0), "tgis_attn_varlen_win: kept first positions need a window");
+    TGIS_CHECK_ARG(!gate || (gate_per_head ? ld_gate >= H
+                                           : (ld_gate >= (int64_t)H * dv && (dtype == TGIS_F32 || (ld_gate % 4 == 0 && ((uintptr_t)gate & 7) == 0)))),
+                   "tgis_attn_varlen_win: the gate needs a row stride >= H (per head) or >= H dv with 8-byte aligned rows");
+    AttnExt ext{nullptr, nullptr, 0, gate, ld_gate,
+                (int)std::min<int64_t>(64, workspace && ((uintptr_t)workspace & 15) == 0 ? workspace_bytes / std::max<int64_t>(1, total_q * H * (int64_t)(dv + 2) * 4) : 0),
+                (float*)workspace, total_q};
+    ext.window = window;
+    ext.keep_first = keep_first;
+    ext.sink = sink;
+    ext.gate_per_head = gate_per_head ? 1 : 0;
+    ext.out_scale = out_scale;
+    return attn_varlen_impl(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, B, out, ld_out, total_q, max_q_len,
+                            max_ctx, H, G, dk, dv, scale, impl, dtype, ext, stream);
 }

@@ -25,7 +25,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, int64_t ld_h, const float* __restrict__ wr,
                                                         const float* __restrict__ wg, int32_t* __restrict__ idx,
                                                         float* __restrict__ weight, float* __restrict__ shared_gate, int W, int E,
-                                                        int k) {
+                                                        int k, const float* __restrict__ router_b, int softmax_top) {
     extern __shared__ float sm[];
     float* hs = sm;          // [W]
     float* logit = sm + W;   // [E + 1]
@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
             for (int c = lane; c < W; c += 64) s += hs[c] * w[c];
         }
         s = wave_sum(s);
-        if (lane == 0) logit[e] = s;
+        if (lane == 0) logit[e] = s + ((router_b && e < E) ? router_b[e] : 0.f);
     }
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -66,8 +66,15 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
             }
             if (best < 0) best = 0;  // NaN logits: still a valid index
             idx[t * k + j] = best;
-            weight[t * k + j] = 1.f / (1.f + expf(-bv));
+            // softmax_top: the chosen logits are softmaxed among themselves below (the first one is the largest)
+            weight[t * k + j] = softmax_top ? bv : 1.f / (1.f + expf(-bv));
             logit[best] = -INFINITY;
+        }
+        if (softmax_top) {
+            const float top = weight[t * k];
+            float sum = 0.f;
+            for (int j = 0; j < k; ++j) sum += expf(weight[t * k + j] - top);
+            for (int j = 0; j < k; ++j) weight[t * k + j] = expf(weight[t * k + j] - top) / sum;
         }
     }
 }
@@ -296,8 +303,9 @@ static bool dtype3(int d) { return d == TGIS_F16 || d == TGIS_BF16 || d == TGIS_
 
 extern "C" int64_t tgis_moe_row_capacity(int64_t n_pairs, int64_t E) { return (n_pairs + E * (TM - 1) + TM - 1) / TM * TM; }
 
-extern "C" int tgis_moe_route(const void* h, int64_t ld_h, const float* router_w, const float* shared_gate_w, int32_t* idx,
-                              float* weight, float* shared_gate, int64_t T, int64_t W, int E, int k, int dtype, void* stream) {
+static int moe_route_impl(const void* h, int64_t ld_h, const float* router_w, const float* shared_gate_w, int32_t* idx,
+                          float* weight, float* shared_gate, int64_t T, int64_t W, int E, int k, int dtype, void* stream,
+                          const float* router_b, int softmax_top) {
     TGIS_CHECK_ARG(h && router_w && idx && weight && (!shared_gate_w || shared_gate), "tgis_moe_route: null tensor");
     TGIS_CHECK_ARG(E >= 1 && k >= 1 && k <= E && W >= 1 && ld_h >= W && dtype3(dtype), "tgis_moe_route: bad arguments");
     const size_t lds = ((size_t)W + E + 1) * sizeof(float);
@@ -305,13 +313,26 @@ extern "C" int tgis_moe_route(const void* h, int64_t ld_h, const float* router_w
     if (T == 0) return TGIS_OK;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == TGIS_F16)
-        hipLaunchKernelGGL(moe_route_kernel<f16>, dim3((unsigned)T), dim3(256), lds, st, (const f16*)h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, (int)W, E, k);
+        hipLaunchKernelGGL(moe_route_kernel<f16>, dim3((unsigned)T), dim3(256), lds, st, (const f16*)h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, (int)W, E, k, router_b, softmax_top);
     else if (dtype == TGIS_BF16)
-        hipLaunchKernelGGL(moe_route_kernel<bf16>, dim3((unsigned)T), dim3(256), lds, st, (const bf16*)h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, (int)W, E, k);
+        hipLaunchKernelGGL(moe_route_kernel<bf16>, dim3((unsigned)T), dim3(256), lds, st, (const bf16*)h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, (int)W, E, k, router_b, softmax_top);
     else
-        hipLaunchKernelGGL(moe_route_kernel<float>, dim3((unsigned)T), dim3(256), lds, st, (const float*)h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, (int)W, E, k);
+        hipLaunchKernelGGL(moe_route_kernel<float>, dim3((unsigned)T), dim3(256), lds, st, (const float*)h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, (int)W, E, k, router_b, softmax_top);
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
+}
+
+extern "C" int tgis_moe_route(const void* h, int64_t ld_h, const float* router_w, const float* shared_gate_w, int32_t* idx,
+                              float* weight, float* shared_gate, int64_t T, int64_t W, int E, int k, int dtype, void* stream) {
+    return moe_route_impl(h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, T, W, E, k, dtype, stream, nullptr, 0);
+}
+
+// The same with a bias on the router logits (router_b [E] fp32 or NULL) and a choice of weights: softmax_top 0: the sigmoid of
+// each chosen logit; 1: the softmax over the chosen logits only.
+extern "C" int tgis_moe_route_ext(const void* h, int64_t ld_h, const float* router_w, const float* router_b, const float* shared_gate_w,
+                                  int softmax_top, int32_t* idx, float* weight, float* shared_gate, int64_t T, int64_t W, int E, int k,
+                                  int dtype, void* stream) {
+    return moe_route_impl(h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, T, W, E, k, dtype, stream, router_b, softmax_top ? 1 : 0);
 }
 
 extern "C" int tgis_moe_align(const int32_t* idx, int64_t n_pairs, int E, int32_t* sorted, int64_t capacity, int32_t* tile_expert,

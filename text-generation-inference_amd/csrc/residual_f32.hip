@@ -434,6 +434,109 @@ void launch_unary(const void* in, int64_t ld_in, const void* other, int64_t ld_o
 
 }  // namespace
 
+// ---- parallel layers with gated residuals and a learned mix over depth ------------------------------------------------
+// One sublayer's result and the gate it passes before it joins the residual stream: delta is a [rows, ld] tensor of TD or the
+// fp32 split-K slabs of the projection that produced it (slabs > 0, ld = their row stride); bias [E] TD is added to it;
+// gate [rows, ld_gate] TD holds logits, gate_bias [E] TD is added to them, and the delta is multiplied by their sigmoid.
+struct GatedDelta {
+    const void* delta;
+    int64_t ld;
+    int slabs;
+    const void* bias;
+    const void* gate;
+    int64_t ld_gate;
+    const void* gate_bias;
+};
+
+template <typename T, int V> struct LdV;
+template <typename T> struct LdV<T, 1> {
+    static __device__ __forceinline__ f32x4 ld(const T* p) { return f32x4{Elem<T>::ld(p), 0.f, 0.f, 0.f}; }
+    static __device__ __forceinline__ void st(T* p, f32x4 v) { *p = cvt_out<T>(v[0]); }
+};
+template <typename T> struct LdV<T, 4> {
+    static __device__ __forceinline__ f32x4 ld(const T* p) { return Vec4<T>::ld(p); }
+    static __device__ __forceinline__ void st(T* p, f32x4 v) { Vec4<T>::st(p, v); }
+};
+
+template <typename TD, int V>
+__device__ __forceinline__ f32x4 gated_delta_at(const GatedDelta& d, int64_t row, int64_t c) {
+    f32x4 v = {};
+    if (d.slabs > 0) {
+        const float* sp = reinterpret_cast<const float*>(d.delta) + ((row >> 5) * d.slabs * 32 + (row & 31)) * d.ld + c;
+        for (int s2 = 0; s2 < d.slabs; ++s2) v += LdV<float, V>::ld(sp + (int64_t)s2 * 32 * d.ld);
+    } else {
+        v = LdV<TD, V>::ld(reinterpret_cast<const TD*>(d.delta) + row * d.ld + c);
+    }
+    if (d.bias) v += LdV<TD, V>::ld(reinterpret_cast<const TD*>(d.bias) + c);
+    if (d.gate) {
+        f32x4 z = LdV<TD, V>::ld(reinterpret_cast<const TD*>(d.gate) + row * d.ld_gate + c);
+        if (d.gate_bias) z += LdV<TD, V>::ld(reinterpret_cast<const TD*>(d.gate_bias) + c);
+#pragma unroll
+        for (int u = 0; u < V; ++u) v[u] *= 1.f / (1.f + expf(-z[u]));
+    }
+    return v;
+}
+
+// One workgroup per row:
+//     v = x + gate_a * a + gate_b * b                       (b optional)
+//     hist[n_prev] = v;   x_out = sum_{j < n_prev} coef[j] hist[j] + coef[n_prev] v        (hist null: x_out = v)
+//     y = x_out / sqrt(mean(x_out^2) + eps) * (pre_w + pre_add)                             (pre_w null: no y)
+// hist entries are hist_stride floats apart.  x_out may alias x (not a hist entry that is still read).
+template <typename TD, typename TY, int V>
+__global__ __launch_bounds__(256) void parallel_residual_kernel(const float* x, GatedDelta a, GatedDelta b, float* hist, int n_prev,
+                                                                int64_t hist_stride, const float* __restrict__ coef, float* x_out,
+                                                                const float* __restrict__ pre_w, float pre_add, TY* __restrict__ y,
+                                                                int64_t E, float eps) {
+    __shared__ float red[16];
+    const int64_t row = blockIdx.x;
+    float ss = 0.f;
+    for (int64_t c = (int64_t)threadIdx.x * V; c < E; c += 256 * V) {
+        f32x4 v = LdV<float, V>::ld(x + row * E + c) + gated_delta_at<TD, V>(a, row, c);
+        if (b.delta) v += gated_delta_at<TD, V>(b, row, c);
+        f32x4 xn = v;
+        if (hist) {
+            LdV<float, V>::st(hist + (int64_t)n_prev * hist_stride + row * E + c, v);
+            xn = v * coef[n_prev];
+            for (int j = 0; j < n_prev; ++j) xn += LdV<float, V>::ld(hist + (int64_t)j * hist_stride + row * E + c) * coef[j];
+        }
+        LdV<float, V>::st(x_out + row * E + c, xn);
+#pragma unroll
+        for (int u = 0; u < V; ++u) ss += xn[u] * xn[u];
+    }
+    if (!pre_w) return;
+    ss = block_sum(ss, red);
+    const float rinv = 1.0f / sqrtf(ss / (float)E + eps);
+    for (int64_t c = (int64_t)threadIdx.x * V; c < E; c += 256 * V) {
+        // the same thread wrote x_out[c .. c + V) above
+        const f32x4 xn = LdV<float, V>::ld(x_out + row * E + c);
+        f32x4 w = LdV<float, V>::ld(pre_w + c);
+#pragma unroll
+        for (int u = 0; u < V; ++u) w[u] = xn[u] * rinv * (w[u] + pre_add);
+        LdV<TY, V>::st(y + row * E + c, w);
+    }
+}
+
+template <typename TD, typename TY>
+void launch_parallel_residual(const float* x, const GatedDelta& a, const GatedDelta& b, float* hist, int n_prev, int64_t hist_stride,
+                              const float* coef, float* x_out, const float* pre_w, float pre_add, void* y, int64_t rows, int64_t E,
+                              float eps, hipStream_t st) {
+    auto al = [](const void* p, int n) { return ((uintptr_t)p % n) == 0; };
+    auto ok = [&](const GatedDelta& d) {
+        if (!d.delta) return true;
+        const int esz = d.slabs > 0 ? 4 : (int)sizeof(TD);
+        return d.ld % 4 == 0 && al(d.delta, 4 * esz) && al(d.bias, 4 * sizeof(TD)) && al(d.gate, 4 * sizeof(TD)) &&
+               al(d.gate_bias, 4 * sizeof(TD)) && (!d.gate || d.ld_gate % 4 == 0);
+    };
+    const bool vec = E % 4 == 0 && ok(a) && ok(b) && al(x, 16) && al(x_out, 16) && al(hist, 16) && hist_stride % 4 == 0 && al(pre_w, 16) &&
+                     al(y, 4 * sizeof(TY));
+    if (vec)
+        hipLaunchKernelGGL((parallel_residual_kernel<TD, TY, 4>), dim3((unsigned)rows), dim3(256), 0, st, x, a, b, hist, n_prev, hist_stride,
+                           coef, x_out, pre_w, pre_add, (TY*)y, E, eps);
+    else
+        hipLaunchKernelGGL((parallel_residual_kernel<TD, TY, 1>), dim3((unsigned)rows), dim3(256), 0, st, x, a, b, hist, n_prev, hist_stride,
+                           coef, x_out, pre_w, pre_add, (TY*)y, E, eps);
+}
+
 static bool dtype3(int d) { return d == TGIS_F16 || d == TGIS_BF16 || d == TGIS_F32; }
 
 extern "C" int tgis_embedding_scaled_f32(const int64_t* ids, const void* table, float* out, int64_t T, int64_t E, int64_t vocab,
@@ -621,6 +724,43 @@ extern "C" int tgis_rms_norm_rows(const void* x, int64_t ld_x, const float* w, v
     TgisTimedScope timed(TGIS_OP_NORM, st);
     TGIS_BY_DTYPE(dtype, hipLaunchKernelGGL(rms_norm_rows_kernel<TT>, dim3((unsigned)cdiv64(rows, 4)), dim3(256), 0, st, (const TT*)x,
                                              ld_x, w, (TT*)y, ld_y, rows, (int)C, eps));
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+// The residual update of a PARALLEL layer (one norm, mixer and feed-forward side by side) with gated residuals and a learned
+// mix over depth, and the next layer's norm, in one launch:
+//     v = x + sigmoid(gate_a + gate_bias_a) * (a + bias_a) + sigmoid(gate_b + gate_bias_b) * (b + bias_b)
+//     hist[n_prev] = v;   x_out = sum_{j <= n_prev} mix[j] hist[j]            (hist NULL: x_out = v)
+//     y = x_out / sqrt(mean(x_out^2) + eps) * (pre_w + pre_add)               (pre_w NULL: none)
+// a / b: [rows, ld] tensors of `dtype`, or (slabs_x > 0) the fp32 split-K slabs of tgis_dense_gemm_partial with ld_x their row
+// stride; b may be NULL (a layer without a feed-forward); biases [E] and gate logits [rows, ld_gate] / gate biases [E] are of
+// `dtype`, each may be NULL.  hist: n_prev + 1 entries of [rows, E] fp32, hist_stride floats apart; mix [n_prev + 1] fp32.
+extern "C" int tgis_parallel_residual_f32(const float* x, const void* a, int64_t ld_a, int slabs_a, const void* bias_a, const void* gate_a,
+                                          int64_t ld_gate_a, const void* gate_bias_a, const void* b, int64_t ld_b, int slabs_b,
+                                          const void* bias_b, const void* gate_b, int64_t ld_gate_b, const void* gate_bias_b, int dtype,
+                                          float* hist, int n_prev, int64_t hist_stride, const float* mix, float* x_out, const float* pre_w,
+                                          float pre_add, void* y, int y_dtype, int64_t rows, int64_t E, float eps, void* stream) {
+    TGIS_CHECK_ARG(x && a && x_out && E > 0 && rows >= 0 && dtype3(dtype), "tgis_parallel_residual_f32: bad arguments");
+    TGIS_CHECK_ARG(ld_a >= E && (!b || ld_b >= E) && (!gate_a || ld_gate_a >= E) && (!gate_b || ld_gate_b >= E) && slabs_a >= 0 && slabs_b >= 0,
+                   "tgis_parallel_residual_f32: bad strides");
+    TGIS_CHECK_ARG(!hist || (mix && n_prev >= 0 && hist_stride >= rows * E), "tgis_parallel_residual_f32: the depth mix needs coefficients and a stride");
+    TGIS_CHECK_ARG(!pre_w || (y && dtype3(y_dtype)), "tgis_parallel_residual_f32: the normed output needs a buffer and a dtype");
+    if (rows == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    TgisTimedScope timed(TGIS_OP_NORM, st);
+    const GatedDelta da{a, ld_a, slabs_a, bias_a, gate_a, ld_gate_a, gate_bias_a};
+    const GatedDelta db{b, ld_b, slabs_b, bias_b, gate_b, ld_gate_b, gate_bias_b};
+#define TGIS_PAR_Y(TD)                                                                                                                  \
+    do {                                                                                                                                \
+        if (y_dtype == TGIS_F16) launch_parallel_residual<TD, f16>(x, da, db, hist, n_prev, hist_stride, mix, x_out, pre_w, pre_add, y, rows, E, eps, st);        \
+        else if (y_dtype == TGIS_BF16) launch_parallel_residual<TD, bf16>(x, da, db, hist, n_prev, hist_stride, mix, x_out, pre_w, pre_add, y, rows, E, eps, st); \
+        else launch_parallel_residual<TD, float>(x, da, db, hist, n_prev, hist_stride, mix, x_out, pre_w, pre_add, y, rows, E, eps, st);                          \
+    } while (0)
+    if (dtype == TGIS_F16) TGIS_PAR_Y(f16);
+    else if (dtype == TGIS_BF16) TGIS_PAR_Y(bf16);
+    else TGIS_PAR_Y(float);
+#undef TGIS_PAR_Y
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
 }

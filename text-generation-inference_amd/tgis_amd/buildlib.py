@@ -19,6 +19,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-tar
 FAMILY_UNITS = {
     "lenisun": ["api", "elementwise", "gemm_dense", "residual_f32", "attn_varlen", "wkv", "moe", "sampler"],
     "senadra": ["api", "elementwise", "gemm_dense", "residual_f32", "attn_varlen", "delta_rule", "sampler"],
+    "mananex": ["api", "elementwise", "gemm_dense", "residual_f32", "attn_varlen", "gated_linear_scan", "moe", "sampler"],
 }
 
 

@@ -55,6 +55,10 @@ class BaseInferenceEngine:
             from tgis_amd.models.custom_modeling.flash_senadra_modeling import SenadraConfig
 
             return SenadraConfig(**raw)
+        if family == "mananex":
+            from tgis_amd.models.custom_modeling.flash_mananex_modeling import MananexConfig
+
+            return MananexConfig(**raw)
         from transformers import AutoConfig
 
         return AutoConfig.from_pretrained(model_path)

@@ -133,6 +133,16 @@ SIGNATURES = {
     "tgis_delta_state_floats": (_c_i64, [_c_int, _c_int]),
     "tgis_delta_scan": (_c_int, [_vp, _c_i64, _vp, _c_i64, _vp, _c_i64, _vp, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _c_i64, _vp, _vp,
                                  _vp, _vp, _c_i64, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_f, _c_f, _c_f, _c_int, _vp]),
+    "tgis_rope_rows_kv_write": (_c_int, [_vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp, _c_i64, _c_int, _c_int, _c_int,
+                                         _c_int, _c_int, _c_int, _vp]),
+    "tgis_attn_varlen_win": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_i64,
+                                      _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int, _vp, _vp, _c_i64, _c_int, _c_f, _vp, _c_i64,
+                                      _c_int, _c_int, _vp]),
+    "tgis_gated_linear_scan": (_c_int, [_vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_i64, _c_f,
+                                        _c_i64, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int, _vp]),
+    "tgis_moe_route_ext": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _c_int, _vp, _vp, _vp, _c_i64, _c_i64, _c_int, _c_int, _c_int, _vp]),
+    "tgis_parallel_residual_f32": (_c_int, [_vp, _vp, _c_i64, _c_int, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _c_int, _vp, _vp, _c_i64, _vp,
+                                            _c_int, _vp, _c_int, _c_i64, _vp, _vp, _vp, _c_f, _vp, _c_int, _c_i64, _c_i64, _c_f, _vp]),
 }
 
 _lib = None
@@ -840,9 +850,11 @@ def _i32(t: Optional[torch.Tensor], what: str):
     return _ptr(t)
 
 
-def embedding_scaled_f32(ids: torch.Tensor, table: torch.Tensor, scale: float) -> torch.Tensor:
+def embedding_scaled_f32(ids: torch.Tensor, table: torch.Tensor, scale: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     assert ids.dtype == torch.int64 and ids.dim() == 1 and table.dim() == 2 and table.is_contiguous()
-    out = torch.empty((ids.shape[0], table.shape[1]), dtype=torch.float32, device=table.device)
+    if out is None:
+        out = torch.empty((ids.shape[0], table.shape[1]), dtype=torch.float32, device=table.device)
+    assert out.dtype == torch.float32 and out.is_contiguous() and out.shape == (ids.shape[0], table.shape[1])
     _check(load_library().tgis_embedding_scaled_f32(_ptr(ids), _ptr(table), _ptr(out), ids.shape[0], table.shape[1],
                                                     table.shape[0], float(scale), dtype_code3(table.dtype), _stream()),
            "tgis_embedding_scaled_f32")
@@ -958,16 +970,22 @@ def moe_row_capacity(n_pairs: int, E: int) -> int:
     return load_library().tgis_moe_row_capacity(n_pairs, E)
 
 
-def moe_route(h, router_w, shared_gate_w, k: int):
-    """(idx int32 [T, k], weight fp32 [T, k], shared gate fp32 [T] or None)."""
+def moe_route(h, router_w, shared_gate_w, k: int, router_b=None, softmax_top: bool = False):
+    """(idx int32 [T, k], weight fp32 [T, k], shared gate fp32 [T] or None).  weight: the sigmoid of each chosen logit, or
+    (softmax_top) the softmax over the chosen logits only; router_b [E] fp32 is added to the logits."""
     T, W = h.shape
     E = router_w.shape[0]
     idx = torch.empty((T, k), dtype=torch.int32, device=h.device)
     weight = torch.empty((T, k), dtype=torch.float32, device=h.device)
     sg = torch.empty((T,), dtype=torch.float32, device=h.device) if shared_gate_w is not None else None
-    _check(load_library().tgis_moe_route(_ptr(h), h.stride(0), _f32(router_w, "router_w"), _f32(shared_gate_w, "shared_gate_w"),
-                                         _ptr(idx), _ptr(weight), _ptr(sg), T, W, E, k, dtype_code3(h.dtype), _stream()),
-           "tgis_moe_route")
+    if router_b is None and not softmax_top:
+        _check(load_library().tgis_moe_route(_ptr(h), h.stride(0), _f32(router_w, "router_w"), _f32(shared_gate_w, "shared_gate_w"),
+                                             _ptr(idx), _ptr(weight), _ptr(sg), T, W, E, k, dtype_code3(h.dtype), _stream()),
+               "tgis_moe_route")
+    else:
+        _check(load_library().tgis_moe_route_ext(_ptr(h), h.stride(0), _f32(router_w, "router_w"), _f32(router_b, "router_b"),
+                                                 _f32(shared_gate_w, "shared_gate_w"), int(softmax_top), _ptr(idx), _ptr(weight), _ptr(sg),
+                                                 T, W, E, k, dtype_code3(h.dtype), _stream()), "tgis_moe_route_ext")
     return idx, weight, sg
 
 
@@ -1181,3 +1199,98 @@ def delta_scan(conv, a, b, gate, A_log, dt_bias, gain, state, tail, proj, state_
         state_slots.shape[0], H, G, dk, dv, taps, float(eps), float(unit_eps), float(q_scale), dtype_code3(a.dtype), _stream()),
         "tgis_delta_scan")
     return out
+
+
+# ---- parallel layers with gated residuals: rotation in the "rows" layout, windowed attention, gated linear scan, update ------
+def rope_rows_kv_write(proj, q_col0: int, k_col0: int, v_col0: int, inv_freq, positions, slots, k_pool, v_pool, H: int, G: int,
+                       dk: int, dv: int, rot_dims: int):
+    """q (in place) and k (into the K pages) of proj [T, ld] rotated in interleaved pairs over their first rot_dims channels; v into
+    the V pages."""
+    assert proj.dim() == 2 and proj.stride(1) == 1 and k_pool.dtype == proj.dtype and v_pool.dtype == proj.dtype
+    assert positions.shape[0] == proj.shape[0] and slots.shape[0] == proj.shape[0]
+    assert rot_dims == 0 or inv_freq.shape[0] >= rot_dims // 2
+    _check(load_library().tgis_rope_rows_kv_write(
+        _ptr(proj), proj.stride(0), q_col0, k_col0, v_col0, _f32(inv_freq, "inv_freq") if rot_dims else None, _i32(positions, "positions"),
+        _i32(slots, "slots"), _ptr(k_pool), _ptr(v_pool), proj.shape[0], H, G, dk, dv, rot_dims, dtype_code3(proj.dtype), _stream()),
+        "tgis_rope_rows_kv_write")
+
+
+def attn_varlen_win(q, k_pool, v_pool, block_tables, ctx_lens, cu_seqlens_q, H: int, G: int, dk: int, dv: int, scale: float,
+                    window: int = 0, keep_first: int = 0, sink=None, gate=None, gate_per_head: bool = False, out_scale: float = 1.0,
+                    out=None, max_q_len: int = 1, max_ctx: int = 1, impl: int = 0, ws: Optional[Workspace] = None):
+    """attn_varlen with a sliding window that keeps the first positions, a sink logit per head (sink [H] fp32), a sigmoid output
+    gate (per head: gate [T, H]; per channel: gate [T, H dv]) and a factor on the output.  out: a [T, H dv] view (unit column
+    stride) of the caller's buffer, or None."""
+    assert q.dim() == 2 and q.stride(1) == 1 and block_tables.dim() == 2
+    T = q.shape[0]
+    assert gate is None or (gate.dtype == q.dtype and gate.stride(1) == 1 and gate.shape == (T, H if gate_per_head else H * dv))
+    assert sink is None or sink.shape[0] == H
+    if out is None:
+        out = torch.empty((T, H * dv), dtype=q.dtype, device=q.device)
+    assert out.shape == (T, H * dv) and out.stride(1) == 1 and out.dtype == q.dtype
+    _check(load_library().tgis_attn_varlen_win(
+        _ptr(q), q.stride(0), _ptr(k_pool), _ptr(v_pool), _i32(block_tables, "block_tables"), block_tables.shape[1],
+        _i32(ctx_lens, "ctx_lens"), _i32(cu_seqlens_q, "cu_seqlens_q"), ctx_lens.shape[0], _ptr(out), out.stride(0), T,
+        max(int(max_q_len), 1), max(int(max_ctx), 1), H, G, dk, dv, float(scale), int(window), int(keep_first), _f32(sink, "sink"),
+        _ptr(gate), gate.stride(0) if gate is not None else 0, int(gate_per_head), float(out_scale),
+        (ws.ptr + 4096) if ws is not None else None, (ws.nbytes - 4096) if ws is not None else 0, impl, dtype_code3(q.dtype), _stream()),
+        "tgis_attn_varlen_win")
+    return out
+
+
+def gated_linear_scan(proj, q_col0: int, f_col0: int, v_col0: int, f_bias, lower, gain, state, state_slots, cu_seqlens_q, positions,
+                      H: int, dk: int, dv: int, eps: float, q_act: bool = True, out_scale: float = 1.0, out=None):
+    """S <- diag(f) S + (1 - f) v^T, o = S^T q per (sequence, head) on columns of proj [T, ld]; f = lower + (1 - lower) *
+    sigmoid(proj_f + f_bias); q = silu(proj_q) if q_act; out = rms_norm(o) * gain * out_scale -> [T, H dv] (or the view `out`)."""
+    assert proj.dim() == 2 and proj.stride(1) == 1
+    T = proj.shape[0]
+    if out is None:
+        out = torch.empty((T, H * dv), dtype=proj.dtype, device=proj.device)
+    assert out.shape == (T, H * dv) and out.stride(1) == 1 and out.dtype == proj.dtype
+    assert state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (H, dk, dv)
+    _check(load_library().tgis_gated_linear_scan(
+        _ptr(proj), proj.stride(0), q_col0, f_col0, v_col0, _f32(f_bias, "f_bias"), _f32(lower, "lower"), _f32(gain, "gain"),
+        _ptr(state), _i32(state_slots, "state_slots"), _i32(cu_seqlens_q, "cu_seqlens_q"), _i32(positions, "positions"), _ptr(out),
+        out.stride(0), float(out_scale), state_slots.shape[0], H, dk, dv, float(eps), int(q_act), dtype_code3(proj.dtype), _stream()),
+        "tgis_gated_linear_scan")
+    return out
+
+
+def _delta_args(d, bias, rows: int, E: int, dtype):
+    """(pointer, row stride, slabs, bias pointer) of a sublayer result: a tensor, or the split-K slabs of its projection."""
+    if d is None:
+        return None, 0, 0, None
+    if isinstance(d, Partial):
+        assert d.shape == (rows, E) and d.dtype == dtype
+        b = d.bias if d.bias is not None else bias
+        assert b is None or (b.dtype == dtype and b.shape[0] == E)
+        return _ptr(d.slabs), d.ld, d.S, _ptr(b)
+    assert d.shape == (rows, E) and d.stride(1) == 1 and d.dtype == dtype
+    assert bias is None or (bias.dtype == dtype and bias.shape[0] == E)
+    return _ptr(d), d.stride(0), 0, _ptr(bias)
+
+
+def parallel_residual_f32(x, a, gate_a, gate_bias_a, b, gate_b, gate_bias_b, act_dtype, hist, n_prev: int, mix, x_out, pre_w,
+                          eps: float, y_dtype, pre_add: float = 0.0, bias_a=None, bias_b=None):
+    """v = x + sigmoid(gate_a + gate_bias_a) a + sigmoid(gate_b + gate_bias_b) b;  hist[n_prev] = v;  x_out = sum_j mix[j] hist[j];
+    returns y = rms_norm(x_out) * (pre_w + pre_add) in y_dtype (None without pre_w).  a / b: tensors of act_dtype or `Partial`
+    split-K slabs (whose bias, if any, is added here); gates are [rows, E] views of logits; hist [>= n_prev + 1, rows, E] fp32
+    or None (then x_out = v)."""
+    rows, E = x.shape
+    assert x.dtype == torch.float32 and x.stride(1) == 1 and x.stride(0) == E and x_out.dtype == torch.float32 and x_out.is_contiguous()
+    for g, gb in ((gate_a, gate_bias_a), (gate_b, gate_bias_b)):
+        assert g is None or (g.dtype == act_dtype and g.stride(1) == 1 and g.shape == (rows, E))
+        assert gb is None or (gb.dtype == act_dtype and gb.shape[0] == E)
+    pa, lda, sa, ba = _delta_args(a, bias_a, rows, E, act_dtype)
+    pb, ldb, sb, bb = _delta_args(b, bias_b, rows, E, act_dtype)
+    if hist is not None:
+        assert hist.dtype == torch.float32 and hist.is_contiguous() and hist.shape[0] > n_prev and tuple(hist.shape[1:]) == (rows, E)
+        assert mix.dtype == torch.float32 and mix.shape[0] == n_prev + 1
+    y = torch.empty((rows, E), dtype=y_dtype, device=x.device) if pre_w is not None else None
+    _check(load_library().tgis_parallel_residual_f32(
+        _ptr(x), pa, lda, sa, ba, _ptr(gate_a), gate_a.stride(0) if gate_a is not None else 0, _ptr(gate_bias_a),
+        pb, ldb, sb, bb, _ptr(gate_b), gate_b.stride(0) if gate_b is not None else 0, _ptr(gate_bias_b), dtype_code3(act_dtype),
+        _ptr(hist), int(n_prev), hist.stride(0) if hist is not None else 0, _f32(mix, "mix") if hist is not None else None, _ptr(x_out),
+        _f32(pre_w, "pre_w"), float(pre_add), _ptr(y), dtype_code3(y_dtype) if y is not None else F32, rows, E, float(eps), _stream()),
+        "tgis_parallel_residual_f32")
+    return y

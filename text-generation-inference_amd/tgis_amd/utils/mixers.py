@@ -17,6 +17,12 @@ argument, so that a model file only maps its config keys and tensor names onto t
                       and to the attention output instead of to every cached token
   DeltaRuleMixer      gated delta rule with a decay per head and key channel, short convolutions in front of q, k and v,
                       low-rank decay and output-gate projections; state in a RecurrentStateCache slot
+  WindowSinkAttention rotated (interleaved pairs, partial) GQA softmax attention with a sliding window that keeps the first
+                      positions, a learned sink logit per head in the denominator and a sigmoid gate per head
+  GatedLinearRecurrence  HGRN2-style linear attention: S <- diag(f) S + (1 - f) v^T with a forget gate bounded below,
+                      o = S^T silu(q), per-head RMS norm; state in a RecurrentStateCache slot
+  SideBySideMixers    several mixers reading the same input through ONE stacked projection, their weighted results through
+                      ONE stacked output projection
   ActivatedMLP        W_down act(W_up h) with the xIELU activation
   TokenSideInput      a slice of a second token embedding, gated by a GELU of a projection of the residual stream itself
 
@@ -126,9 +132,13 @@ class WkvMixer:
 class GatedUnit:
     """mode "silu": silu(g) * u.  mode "clamped": g = min(g, limit), u = clamp(u, +-limit), g * sigmoid(alpha g) * (u + 1)."""
 
-    def __init__(self, weights, prefix: str, mode: str = "silu", alpha: float = 1.0, limit: float = 0.0):
+    def __init__(self, weights, prefix: str, mode: str = "silu", alpha: float = 1.0, limit: float = 0.0, bias: bool = False):
+        """bias: the three projections have biases (`<name>.b`)."""
         self.gate_up = load_stacked_linear(weights, [f"{prefix}.gate", f"{prefix}.up"])
         self.down = load_linear(weights, f"{prefix}.down")
+        if bias:
+            self.gate_up.bias = torch.cat([weights.get_tensor(f"{prefix}.gate.b"), weights.get_tensor(f"{prefix}.up.b")]).contiguous()
+            self.down.bias = weights.get_tensor(f"{prefix}.down.b").contiguous()
         self.ff = self.gate_up.out_features // 2
         self.mode = {"silu": 0, "clamped": 1}[mode]
         self.alpha, self.limit = float(alpha), float(limit)
@@ -157,9 +167,14 @@ class GatedUnit:
 
 
 class RoutedExperts:
-    def __init__(self, weights, prefix: str, experts: int, top: int, shared: bool):
+    def __init__(self, weights, prefix: str, experts: int, top: int, shared: bool, router_bias: bool = False,
+                 softmax_top: bool = False, weight_on_input: bool = True):
+        """softmax_top: the routing weights are the softmax over the chosen logits (else the sigmoid of each);
+        weight_on_input: the weight scales the expert's input (else its output); router_bias: `<prefix>.router.b`."""
         self.E, self.k = experts, top
+        self.softmax_top, self.weight_on_input = bool(softmax_top), bool(weight_on_input)
         self.router = _f32(weights.get_tensor(f"{prefix}.router"))
+        self.router_b = _f32(weights.get_tensor(f"{prefix}.router.b")) if router_bias else None
         pad8 = lambda n: (n + 7) // 8 * 8
         gate = [weights.get_tensor(f"{prefix}.e{e}.gate") for e in range(experts)]
         ff, W = gate[0].shape
@@ -177,15 +192,16 @@ class RoutedExperts:
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         T, W = h.shape
-        idx, weight, sg = native.moe_route(h, self.router, self.shared_gate, self.k)
+        idx, weight, sg = native.moe_route(h, self.router, self.shared_gate, self.k, self.router_b, self.softmax_top)
         sorted_, tile_expert, pos, n_tiles = native.moe_align(idx, self.E)
         cap = sorted_.shape[0]
         hp = h if self.Wp == W else torch.nn.functional.pad(h, (0, self.Wp - W))
         act = native.moe_gemm(hp, self.w_gate_up, self.ff, tile_expert, n_tiles, cap, sorted_=sorted_, pair_div=self.k,
-                              pair_scale=weight.view(-1), glu_act=True)
+                              pair_scale=weight.view(-1) if self.weight_on_input else None, glu_act=True)
         rows = native.moe_gemm(act, self.w_down, W, tile_expert, n_tiles, cap)
         shared = self.shared(h) if self.shared is not None else None
-        return native.moe_combine(rows, pos, self.k, T, shared=shared, shared_gate=sg)
+        return native.moe_combine(rows, pos, self.k, T, pair_weight=None if self.weight_on_input else weight.view(-1),
+                                  shared=shared, shared_gate=sg)
 
     __call__ = forward
 
@@ -342,6 +358,125 @@ class DeltaRuleMixer:
                                 step.state_slots, step.cu_seqlens_q, position_ids, self.H, self.G, self.dk, self.dv, self.taps,
                                 self.eps, self.unit_eps, self.dk ** -0.5)
         return self.o(out, partial=self.defer)
+
+
+def load_stacked_blocks(weights, names, align: int = 8):
+    """Several [out_i, in] weights that read the same input as one GEMM whose every block starts on a multiple of `align`
+    output columns (zero rows between them) and whose width is one too: (FastLinear, [first column of each block])."""
+    parts, cols, at = [], [], 0
+    for n in names:
+        w = weights.get_tensor(n)
+        cols.append(at)
+        pad = -w.shape[0] % align
+        parts.append(w)
+        if pad:
+            parts.append(w.new_zeros((pad, w.shape[1])))
+        at += w.shape[0] + pad
+    return FastLinear(torch.cat(parts, dim=0).contiguous(), None), cols
+
+
+class WindowSinkAttention:
+    """GQA softmax attention: q, k rotated in interleaved pairs (2i, 2i + 1) over their first rot_dims channels by
+    position * rot_base^(-2i / rot_dims); position i sees j <= i iff i - j < window or j < keep_first (window 0: plain causal);
+    the denominator of head h also holds exp(sink[h]) (`<prefix>.sink`, optional); head h's output is multiplied by
+    sigmoid(W_g h)[h] (`<prefix>.g`, optional).  The mixer reads columns of a projection its owner made (`in_names` are the
+    weights to stack, in this order) and writes its heads into the owner's buffer."""
+
+    def __init__(self, weights, prefix: str, layer_id: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
+                 window: int = 0, keep_first: int = 0, rot_base: float = 10000.0, rot_dims: int = 0):
+        self.layer_id = layer_id
+        self.H, self.G, self.dk, self.dv = heads, kv_heads, dim, vdim
+        _widths_ok_for_pages(dim, vdim)
+        if heads % kv_heads or rot_dims % 2 or rot_dims > dim:
+            raise ValueError(f"{prefix}: {heads} heads on {kv_heads} kv heads, {rot_dims} rotated of {dim} channels")
+        self.scale, self.window, self.keep_first = float(scale), int(window), int(keep_first) if window else 0
+        self.rot_dims = int(rot_dims)
+        self.has_gate = weights.has(f"{prefix}.g")
+        self.in_names = [f"{prefix}.{n}" for n in (("q", "k", "v", "g") if self.has_gate else ("q", "k", "v"))]
+        self.out_name, self.out_width = f"{prefix}.o", heads * vdim
+        self.sink = _f32(weights.get_tensor(f"{prefix}.sink")) if weights.has(f"{prefix}.sink") else None
+        dev = weights.device
+        self.inv_freq = rotary_inverse_frequencies(rot_base, self.rot_dims, dev) if self.rot_dims else None
+        self.kv_shape = (kv_heads, dim, vdim)
+        self.state_shape = None
+
+    def run(self, proj: torch.Tensor, cols, position_ids, step, out: torch.Tensor, out_scale: float = 1.0):
+        """proj [T, ld] with this mixer's blocks at columns `cols` (one per in_name); out [T, H dv] (a view)."""
+        cache = step.cache
+        k_pool, v_pool = cache.k_pool(self.layer_id), cache.v_pool(self.layer_id)
+        native.rope_rows_kv_write(proj, cols[0], cols[1], cols[2], self.inv_freq, position_ids, step.slots, k_pool, v_pool, self.H,
+                                  self.G, self.dk, self.dv, self.rot_dims)
+        gate = proj[:, cols[3]:cols[3] + self.H] if self.has_gate else None
+        native.attn_varlen_win(proj[:, cols[0]:cols[0] + self.H * self.dk], k_pool, v_pool, step.block_tables, step.ctx_lens,
+                               step.cu_seqlens_q, self.H, self.G, self.dk, self.dv, self.scale, window=self.window,
+                               keep_first=self.keep_first, sink=self.sink, gate=gate, gate_per_head=True, out_scale=out_scale, out=out,
+                               max_q_len=step.max_q_len, max_ctx=step.max_ctx, ws=workspace(proj.device))
+
+
+class GatedLinearRecurrence:
+    """Per head S <- diag(f) S + (1 - f) v^T, o = S^T q with q = silu(W_q h), v = W_v h and the forget gate
+    f = l + (1 - l) sigmoid(W_f h + b) bounded below by l (`.lower`), one per head and key channel; o is RMS-normed per head
+    with one gain for all heads (`.norm`).  Gates, state and read-out are fp32.  Reads columns of its owner's projection."""
+
+    def __init__(self, weights, prefix: str, layer_id: int, heads: int, dim: int, vdim: int, eps: float):
+        self.layer_id = layer_id
+        self.H, self.dk, self.dv, self.eps = heads, dim, vdim, float(eps)
+        if dim > 256 or vdim > 256:
+            raise NotImplementedError(f"the gated linear scan serves heads of up to 256 x 256 (got {dim} x {vdim})")
+        self.in_names = [f"{prefix}.{n}" for n in ("q", "f", "v")]
+        self.out_name, self.out_width = f"{prefix}.o", heads * vdim
+        self.f_bias = _f32(weights.get_tensor(f"{prefix}.f.b")) if weights.has(f"{prefix}.f.b") else None
+        self.lower = _f32(weights.get_tensor(f"{prefix}.lower")) if weights.has(f"{prefix}.lower") else None
+        self.gain = _f32(weights.get_tensor(f"{prefix}.norm"))
+        self.kv_shape = None
+        # a slot holds the heads' matrices [H, dk, dv]; nothing else is remembered (a one-float placeholder)
+        self.state_shape = {"matrix": (heads, dim, vdim), "memory": (1,)}
+
+    def run(self, proj: torch.Tensor, cols, position_ids, step, out: torch.Tensor, out_scale: float = 1.0):
+        native.gated_linear_scan(proj, cols[0], cols[1], cols[2], self.f_bias, self.lower, self.gain, step.state.state[self.layer_id],
+                                 step.state_slots, step.cu_seqlens_q, position_ids, self.H, self.dk, self.dv, self.eps, q_act=True,
+                                 out_scale=out_scale, out=out)
+
+
+class SideBySideMixers:
+    """Mixers that read the same input and whose results are added with fixed weights: y = sum_m scale_m W_o,m mixer_m(h).
+    Everything that reads h — the mixers' input projections and whatever else the owner names (`extra_in`: gates of the
+    residual, ...) — is ONE stacked GEMM; the mixers write their heads, already scaled, side by side into one buffer, and the
+    output projections are ONE GEMM over it (its split-K sum may be left to the residual update behind it)."""
+
+    def __init__(self, weights, mixers, scales, extra_in=()):
+        self.mixers, self.scales = list(mixers), [float(s) for s in scales]
+        names = [n for m in self.mixers for n in m.in_names] + list(extra_in)
+        self.proj, cols = load_stacked_blocks(weights, names, align=8)
+        self.cols, at = [], 0
+        for m in self.mixers:
+            self.cols.append(cols[at:at + len(m.in_names)])
+            at += len(m.in_names)
+        self.extra_cols = dict(zip(extra_in, cols[at:]))
+        # heads side by side, every mixer's block on a multiple of 8 columns; the output weight gets zero columns there
+        self.out_cols, parts, at = [], [], 0
+        for m in self.mixers:
+            w = weights.get_tensor(m.out_name)
+            pad = -w.shape[1] % 8
+            self.out_cols.append(at)
+            parts.append(w)
+            if pad:
+                parts.append(w.new_zeros((w.shape[0], pad)))
+            at += w.shape[1] + pad
+        self.out_width = at
+        self.padded = any(m.out_width % 8 for m in self.mixers)
+        self.o = FastLinear(torch.cat(parts, dim=1).contiguous(), None)
+        self.defer = can_defer(self.o)
+
+    def forward(self, h: torch.Tensor, position_ids, step):
+        """(y [T, W] or its split-K slabs, proj): proj holds the extra blocks at self.extra_cols[name]."""
+        proj = self.proj(h)
+        T = h.shape[0]
+        alloc = torch.zeros if self.padded else torch.empty
+        heads = alloc((T, self.out_width), dtype=h.dtype, device=h.device)
+        for m, cols, c0, sc in zip(self.mixers, self.cols, self.out_cols, self.scales):
+            m.run(proj, cols, position_ids, step, heads[:, c0:c0 + m.out_width], out_scale=sc)
+        return self.o(heads, partial=self.defer), proj
 
 
 def _softplus(z: float) -> float:
