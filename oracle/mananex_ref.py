@@ -97,6 +97,11 @@ def window_sink_attention(h, pos, p: Dict[str, torch.Tensor], m: dict, past_k=No
     return out.reshape(T, H * dv) @ p["o"].T, k, v
 
 
+# when a list: gated_linear_recurrence appends, per token, the smallest |S^T q| / (|S|^T |q|) over the heads: how much of the
+# read-out is left after its terms cancel (the per-head norm that follows divides by it)
+READOUT_CONDITION = None
+
+
 def forget_gate(z, lower):
     """f = l + (1 - l) sigmoid(z): a forget gate that cannot fall below l."""
     return lower + (1.0 - lower) * torch.sigmoid(z)
@@ -108,6 +113,9 @@ def gated_linear_recurrence(q, f, v, S):
     for t in range(q.shape[0]):
         S = S * f[t][:, :, None] + (1.0 - f[t])[:, :, None] * v[t][:, None, :]
         out[t] = torch.einsum("hkv,hk->hv", S, q[t])
+        if READOUT_CONDITION is not None:
+            bound = torch.einsum("hkv,hk->hv", S.abs(), q[t].abs())
+            READOUT_CONDITION.append(float((out[t].norm(dim=-1) / bound.norm(dim=-1).clamp_min(1e-300)).min()))
     return out, S
 
 
@@ -133,11 +141,42 @@ def gated_unit(h, p, prefix=""):
     return y + p[prefix + "down.b"] if prefix + "down.b" in p else y
 
 
+# when a list: route_top_softmax appends, per call, the smallest gap between a chosen and an unchosen logit (how close the
+# routing of these tokens is to falling the other way)
+ROUTER_MARGINS = None
+
+
 def route_top_softmax(h, p, top: int):
     """(indices [T, top], weights [T, top]): the largest logits, softmaxed among themselves."""
     z = h @ p["router"].T + p["router.b"]
     val, idx = torch.topk(z, top, dim=-1)
+    if ROUTER_MARGINS is not None and top < z.shape[-1]:
+        ROUTER_MARGINS.append(float((val[:, -1] - torch.topk(z, top + 1, dim=-1).values[:, -1]).min()))
     return idx, torch.softmax(val, -1)
+
+
+def clear_cut_tokens(config, tensors, n: int, seed: int, margin: float = 0.3, condition: float = 0.1) -> List[int]:
+    """n random tokens, each drawn again until no router of the model is within `margin` of choosing other experts for it and
+    no head's read-out of the recurrence cancels to less than `condition` of its terms before it is normed: what a
+    reduced-precision run computes for them differs from this restatement by rounding, not by a decision or a division that
+    rounding tips."""
+    global ROUTER_MARGINS, READOUT_CONDITION
+    g = torch.Generator().manual_seed(seed)
+    state, toks = new_state(config), []
+    try:
+        while len(toks) < n:
+            for _ in range(50):
+                t = int(torch.randint(0, config["vocab"], (1,), generator=g))
+                trial = {"len": state["len"], "layers": list(state["layers"])}
+                ROUTER_MARGINS, READOUT_CONDITION = [], []
+                advance(config, tensors, [t], trial)
+                if all(m >= margin for m in ROUTER_MARGINS) and all(c >= condition for c in READOUT_CONDITION):
+                    break
+            state = trial
+            toks.append(t)
+    finally:
+        ROUTER_MARGINS = READOUT_CONDITION = None
+    return toks
 
 
 def expert_mixture(h, p, f: dict):

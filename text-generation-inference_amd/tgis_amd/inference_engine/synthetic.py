@@ -259,3 +259,64 @@ def senadra_tensors(config, seed: int, device="cpu", dtype=torch.bfloat16, low_r
     vec("final.norm", W, 1.0)
     lin("head", config.vocab, W)
     return t
+
+
+def mananex_tensors(config, seed: int, device="cpu", dtype=torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """Seeded full Mananex checkpoint in the family's tensor naming for a `MananexConfig`: N(0, 1 / fan_in) projections, norm
+    gains around zero (offsets from one), lower bounds of the forget gates spread over (0, 1), depth-mix coefficients that
+    weigh the newest entry most."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    W = config.width
+    t: Dict[str, torch.Tensor] = {}
+
+    def lin(name, n, k, gain=1.0):
+        t[name] = (torch.randn(n, k, generator=g, device=device) * gain * k ** -0.5).to(dtype)
+
+    def vec(name, n, mean=0.0, std=0.05):
+        t[name] = (mean + torch.randn(n, generator=g, device=device) * std).to(dtype)
+
+    t["embed"] = torch.randn(config.vocab, W, generator=g, device=device).to(dtype)
+    for i, lay in enumerate(config.layers):
+        m = lay["mixer"]
+        vec(f"l{i}.norm1", W)
+        a, p = m["left"], f"l{i}.mix.left"
+        H, dk = a["heads"], a["dim"]
+        G, dv = a.get("kv_heads", H), a.get("vdim", dk)
+        lin(f"{p}.q", H * dk, W)
+        lin(f"{p}.k", G * dk, W)
+        lin(f"{p}.v", G * dv, W)
+        vec(f"{p}.sink", H, 0.0, 1.0)
+        lin(f"{p}.g", H, W)
+        lin(f"{p}.o", W, H * dv)
+        r, p = m["right"], f"l{i}.mix.right"
+        Hr, dkr, dvr = r["heads"], r["dim"], r.get("vdim", r["dim"])
+        lin(f"{p}.q", Hr * dkr, W)
+        lin(f"{p}.f", Hr * dkr, W)
+        vec(f"{p}.f.b", Hr * dkr, 0.5, 1.0)
+        t[f"{p}.lower"] = (torch.rand(Hr * dkr, generator=g, device=device) * 0.9).to(dtype)
+        lin(f"{p}.v", Hr * dvr, W)
+        vec(f"{p}.norm", dvr, 1.0)
+        lin(f"{p}.o", W, Hr * dvr)
+        lin(f"l{i}.rg1", W, W)
+        vec(f"l{i}.rg1.b", W, 0.5, 0.5)
+        f = lay.get("mlp")
+        if f:
+            q = f"l{i}.mlp"
+            lin(f"l{i}.rg2", W, W)
+            vec(f"l{i}.rg2.b", W, 0.5, 0.5)
+            if f["kind"] == "dense":
+                for n_, (o_, i_) in (("gate", (f["ff"], W)), ("up", (f["ff"], W)), ("down", (W, f["ff"]))):
+                    lin(f"{q}.{n_}", o_, i_)
+                    vec(f"{q}.{n_}.b", o_, 0.0, 0.1)
+            else:
+                for e in range(f["router"]["experts"]):
+                    lin(f"{q}.e{e}.gate", f["expert"]["ff"], W)
+                    lin(f"{q}.e{e}.up", f["expert"]["ff"], W)
+                    lin(f"{q}.e{e}.down", W, f["expert"]["ff"])
+                lin(f"{q}.router", f["router"]["experts"], W)
+                vec(f"{q}.router.b", f["router"]["experts"], 0.0, 0.5)
+        c = torch.randn(i + 2, generator=g, device=device) * (0.3 / (i + 2))
+        c[-1] += 0.9
+        t[f"l{i}.dwa"] = c.to(dtype)
+    vec("final.norm", W)
+    return t
