@@ -438,6 +438,24 @@ def senadra_layers(variant, width, layers, heads, kv_heads, dim, ff):
     return out
 
 
+def mananex_layers(variant, width, layers, heads, kv_heads, dim, ff):
+    """"mananex_dense": every layer the two mixers side by side (attention with a window longer than any context here, so that
+    the cache bytes equal Llama's, and a recurrence of width / 256 heads of 64 x 128) + the gated unit with biases.
+    "mananex": a window of 512 positions that keeps the first 4, and every second feed-forward a mixture of 8 experts of
+    ff / 4, top 2 — the design as it is meant."""
+    out = []
+    for i in range(layers):
+        mlp = {"kind": "dense", "ff": ff}
+        if variant == "mananex" and i % 2 == 1:
+            mlp = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 8, "top": 2}}
+        window = 512 if variant == "mananex" else 8192
+        out.append({"type": "parallel", "mlp": mlp,
+                    "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                       "mask": {"size": window, "keep_first": 4}, "rot": {"base": 10000.0, "dims": dim}},
+                              "right": {"heads": max(1, width // 256), "dim": 64, "vdim": 128}, "left_scale": 1.0, "right_scale": 1.0}})
+    return out
+
+
 def bench_hybrid(args):
     """Prefill and decode throughput + per-kernel-class device time (HIP events, eager pass) of Lenisun variants and of
     Llama at the same size, through the same entry points (from_pb -> generate_token).  One JSON line."""
@@ -470,6 +488,13 @@ def bench_hybrid(args):
                               num_attention_heads=heads, num_key_value_heads=kv_heads, rms_norm_eps=1e-5)
             tensors = llama_tensors(cfg, None, seed=1234, device=device, dtype=dtype)
             n_attn, n_scan = layers, 0
+        elif name.startswith("mananex"):
+            from tgis_amd.inference_engine.synthetic import mananex_tensors
+            from tgis_amd.models.custom_modeling.flash_mananex_modeling import MananexConfig
+
+            cfg = MananexConfig(width=width, vocab=vocab, norm={"eps": 1e-5}, layers=mananex_layers(name, width, layers, heads, kv_heads, dim, ff))
+            tensors = mananex_tensors(cfg, seed=1234, device=device, dtype=dtype)
+            n_attn = n_scan = layers
         elif name.startswith("senadra"):
             cfg = SenadraConfig(width=width, vocab=vocab, norm={"eps": 1e-5}, residual_mult=0.25, token_side={"dim": 64},
                                 logit_softcap=25.0, layers=senadra_layers(name, width, layers, heads, kv_heads, dim, ff))
@@ -539,7 +564,8 @@ def bench_hybrid(args):
             ctx_now = L_in + W + K + 2
             if "attention" in kern:
                 # bytes one attention launch has to read: every cached key and value of the batch once
-                by = B * ctx_now * kv_heads * 2 * dim * 2
+                keys = min(ctx_now, 512 + 4 + 32) if name == "mananex" else ctx_now  # a window, its kept positions, a page's slack
+                by = B * keys * kv_heads * 2 * dim * 2
                 kern["attention"]["algorithmic_bytes"] = by
                 kern["attention"]["frac_of_hbm_peak"] = round(by / (kern["attention"]["us_per_launch"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)
             rec["decode"] = {"batch": B, "ctx": ctx_now, "ms_per_step": round(dt * 1e3, 4), "tokens_per_s": round(B / dt, 1),
@@ -575,7 +601,7 @@ def main():
     ap.add_argument("--hybrid", choices=sorted(HYBRID_SIZES), default=None,
                     help="instead of the default workload: Lenisun / Senadra variants beside Llama at this size (prefill + decode)")
     ap.add_argument("--hybrid-models", default="llama,attn,mixed",
-                    help="comma list of llama, attn, mixed (Lenisun), senadra_attn, senadra")
+                    help="comma list of llama, attn, mixed (Lenisun), senadra_attn, senadra, mananex_dense, mananex")
     ap.add_argument("--prefill-batch", type=int, default=4)
     ap.add_argument("--prefill-len", type=int, default=1024)
     ap.add_argument("--prefill-reps", type=int, default=3)

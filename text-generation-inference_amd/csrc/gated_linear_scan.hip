@@ -9,87 +9,150 @@
 // step that starts at position 0 starts from zeros whatever the slot holds.  Gates, (1 - f), the state and the read-out are
 // fp32 whatever the activation dtype T of the projections is.
 //
-// Workgroup = (sequence, head) = dv_pad x 4 threads: a quad of neighbouring lanes shares column j of S, lane q of the quad
-// keeps rows q RPL .. q RPL + RPL - 1 in registers.  Tokens go through LDS in stages of TS: the stage's q and f rows (activated,
-// fp32, one padded segment per row group so that the four groups' 16-byte reads fall into different banks) and v rows; per token
-// a lane does RPL fused updates s = v + f (s - v) and RPL products for the read-out, the quad adds up by two lane exchanges, and
-// the stage's outputs wait in LDS for the norm, which a wave does per token once the stage is through.
+// Workgroup = (sequence, head) = dv_pad x 4 threads: a quad of neighbouring lanes shares column j of S, lane q of the quad keeps
+// rows q RPL .. q RPL + RPL - 1 in registers.  Tokens go through LDS in stages of `ts`: the stage's q and f rows (activated,
+// fp32, one padded segment per row group so that the four groups' 16-byte reads fall into different banks) and v rows, in two
+// buffers.  A thread asks for its share of the NEXT stage's projections before it works through the current one (per token RPL
+// updates s = f s + (1 - f) v and RPL products for the read-out; the quad adds up by two data-parallel-primitive moves), and activates and
+// stores them afterwards: the trip to memory is hidden behind the arithmetic.  The stage's outputs wait in LDS for the norm,
+// which a wave does per token once the stage is through.
+#include <algorithm>
 #include "common.h"
 
 namespace {
 
-constexpr int TS = 16;   // tokens per stage
 constexpr int SEG_PAD = 4;  // floats between the row groups' segments
+constexpr int PFQ = 2;      // (q, f) pairs and
+constexpr int PFV = 4;      // values of the next stage that a thread holds in registers: ts dk <= PFQ threads, ts dv <= PFV threads
 
 template <typename T> __device__ __forceinline__ float ldf(const T* p) { return (float)*p; }
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-z)); }
 
-template <typename T, int RPL>
-__global__ __launch_bounds__(1024) void gated_linear_scan_kernel(
-    const T* __restrict__ proj, int64_t ld, int64_t q_col0, int64_t f_col0, int64_t v_col0, const float* __restrict__ f_bias,
-    const float* __restrict__ lower, const float* __restrict__ gain, float* __restrict__ state, const int32_t* __restrict__ state_slots,
-    const int32_t* __restrict__ cu_q, const int32_t* __restrict__ positions, T* __restrict__ out, int64_t ld_out, float out_scale, int H,
-    int dk, int dv, int dv_pad, float eps, int q_act) {
+struct ScanArgs {
+    const void* proj;
+    int64_t ld, q_col0, f_col0, v_col0;
+    const float* f_bias;
+    const float* lower;
+    const float* gain;
+    float* state;
+    const int32_t* state_slots;
+    const int32_t* cu_q;
+    const int32_t* positions;
+    void* out;
+    int64_t ld_out;
+    float out_scale;
+    int H, dk, dv, dv_pad, ts;
+    float eps;
+    int q_act;
+};
+
+template <typename T, int RPL, int MAXT>
+__global__ __launch_bounds__(MAXT) void gated_linear_scan_kernel(ScanArgs a) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
     constexpr int SEG = RPL + SEG_PAD, ROW = 4 * SEG;
-    float* qs = smem;                       // [TS][ROW]
-    float* fs = qs + TS * ROW;              // [TS][ROW]
-    float* vs = fs + TS * ROW;              // [TS][dv_pad]
-    float* os = vs + TS * dv_pad;           // [TS][dv_pad]
+    const int ts = a.ts, dk = a.dk, dv = a.dv, dv_pad = a.dv_pad;
+    float* qs = smem;                        // [2][ts][ROW]
+    float* fs = qs + 2 * ts * ROW;           // [2][ts][ROW]
+    float* vs = fs + 2 * ts * ROW;           // [2][ts][dv_pad]
+    float* os = vs + 2 * ts * dv_pad;        // [ts][dv_pad]
     const int b = blockIdx.x, h = blockIdx.y;
     const int tid = threadIdx.x, j = tid >> 2, qd = tid & 3;
-    const int t0 = cu_q[b], qlen = cu_q[b + 1] - t0;
+    const int t0 = a.cu_q[b], qlen = a.cu_q[b + 1] - t0;
     if (qlen <= 0) return;
-    const bool fresh = positions[t0] == 0;
-    float* S = state + ((int64_t)state_slots[b] * H + h) * (int64_t)dk * dv;
+    const int nthreads = blockDim.x;
+    const bool fresh = a.positions[t0] == 0;
+    const T* proj = reinterpret_cast<const T*>(a.proj);
+    float* S = a.state + ((int64_t)a.state_slots[b] * a.H + h) * (int64_t)dk * dv;
     float s[RPL];
 #pragma unroll
     for (int r = 0; r < RPL; ++r) {
         const int i = qd * RPL + r;
         s[r] = (!fresh && i < dk && j < dv) ? S[(int64_t)i * dv + j] : 0.f;
     }
-    const int nthreads = blockDim.x, wave = tid >> 6, lane = tid & 63, nw = nthreads >> 6;
-    for (int base = 0; base < qlen; base += TS) {
-        const int n = min(TS, qlen - base);
-        __syncthreads();  // the stage before is consumed (its outputs normed)
-        for (int e = tid; e < n * 4 * RPL; e += nthreads) {
-            const int tt = e / (4 * RPL), i = e - tt * (4 * RPL);
-            float qv = 0.f, fv = 1.f;  // rows past dk: the state stays zero and is never read
-            if (i < dk) {
-                const T* row = proj + (int64_t)(t0 + base + tt) * ld;
-                qv = ldf(row + q_col0 + (int64_t)h * dk + i);
-                if (q_act) qv = qv * sigmoid_f(qv);
-                const float z = ldf(row + f_col0 + (int64_t)h * dk + i) + (f_bias ? f_bias[h * dk + i] : 0.f);
-                const float lo = lower ? lower[h * dk + i] : 0.f;
-                fv = lo + (1.f - lo) * sigmoid_f(z);
+    // rows past dk and columns past dv of both buffers: f = 1, q = 0, v = 0 (their state stays zero and is never read)
+    for (int e = tid; e < 2 * ts * ROW; e += nthreads) {
+        qs[e] = 0.f;
+        fs[e] = 1.f;
+    }
+    for (int e = tid; e < 2 * ts * dv_pad; e += nthreads) vs[e] = 0.f;
+    T qr[PFQ], fr[PFQ], vr[PFV];
+    // tokens [first, first + n) of the sequence: this thread's share of their projections, as they are
+    auto fetch = [&](int first, int n) {
+#pragma unroll
+        for (int u = 0; u < PFQ; ++u) {
+            const int e = tid + u * nthreads;
+            if (e < n * dk) {
+                const int tt = e / dk, i = e - tt * dk;
+                const T* row = proj + (int64_t)(t0 + first + tt) * a.ld + (int64_t)h * dk + i;
+                qr[u] = row[a.q_col0];
+                fr[u] = row[a.f_col0];
             }
-            const int at = tt * ROW + (i / RPL) * SEG + (i % RPL);
-            qs[at] = qv;
-            fs[at] = fv;
         }
-        for (int e = tid; e < n * dv_pad; e += nthreads) {
-            const int tt = e / dv_pad, c = e - tt * dv_pad;
-            vs[e] = c < dv ? ldf(proj + (int64_t)(t0 + base + tt) * ld + v_col0 + (int64_t)h * dv + c) : 0.f;
+#pragma unroll
+        for (int u = 0; u < PFV; ++u) {
+            const int e = tid + u * nthreads;
+            if (e < n * dv) {
+                const int tt = e / dv, c = e - tt * dv;
+                vr[u] = proj[(int64_t)(t0 + first + tt) * a.ld + a.v_col0 + (int64_t)h * dv + c];
+            }
         }
-        __syncthreads();
+    };
+    // ... activated and stored into one stage buffer
+    auto commit = [&](int n, float* qb, float* fb, float* vb) {
+#pragma unroll
+        for (int u = 0; u < PFQ; ++u) {
+            const int e = tid + u * nthreads;
+            if (e < n * dk) {
+                const int tt = e / dk, i = e - tt * dk;
+                float qv = (float)qr[u];
+                if (a.q_act) qv = qv * sigmoid_f(qv);
+                const float z = (float)fr[u] + (a.f_bias ? a.f_bias[h * dk + i] : 0.f);
+                const float lo = a.lower ? a.lower[h * dk + i] : 0.f;
+                const int at = tt * ROW + (i / RPL) * SEG + (i % RPL);
+                qb[at] = qv;
+                fb[at] = lo + (1.f - lo) * sigmoid_f(z);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < PFV; ++u) {
+            const int e = tid + u * nthreads;
+            if (e < n * dv) {
+                const int tt = e / dv, c = e - tt * dv;
+                vb[tt * dv_pad + c] = (float)vr[u];
+            }
+        }
+    };
+    fetch(0, min(ts, qlen));
+    __syncthreads();  // the buffers are filled with their neutral values
+    commit(min(ts, qlen), qs, fs, vs);
+    __syncthreads();
+    const int wave = tid >> 6, lane = tid & 63, nw = nthreads >> 6;
+    T* out = reinterpret_cast<T*>(a.out);
+    int buf = 0;
+    for (int base = 0; base < qlen; base += ts, buf ^= 1) {
+        const int n = min(ts, qlen - base);
+        const int n_next = min(ts, qlen - base - ts);
+        if (n_next > 0) fetch(base + ts, n_next);
+        const float* qb = qs + buf * ts * ROW + qd * SEG;
+        const float* fb = fs + buf * ts * ROW + qd * SEG;
+        const float* vb = vs + buf * ts * dv_pad + j;
+#pragma unroll 1
         for (int tt = 0; tt < n; ++tt) {
-            const float vj = vs[tt * dv_pad + j];
-            const float* qrow = qs + tt * ROW + qd * SEG;
-            const float* frow = fs + tt * ROW + qd * SEG;
+            const float vj = vb[tt * dv_pad];
             float acc = 0.f;
 #pragma unroll
             for (int r4 = 0; r4 < RPL; r4 += 4) {
-                const f32x4 f4 = *reinterpret_cast<const f32x4*>(frow + r4);
-                const f32x4 q4 = *reinterpret_cast<const f32x4*>(qrow + r4);
+                const f32x4 f4 = *reinterpret_cast<const f32x4*>(fb + tt * ROW + r4);
+                const f32x4 q4 = *reinterpret_cast<const f32x4*>(qb + tt * ROW + r4);
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    // f s + (1 - f) v
-                    s[r4 + u] = f4[u] * s[r4 + u] + (1.f - f4[u]) * vj;
-                    acc += s[r4 + u] * q4[u];
+                    s[r4 + u] = fmaf(f4[u], s[r4 + u], (1.f - f4[u]) * vj);
+                    acc = fmaf(s[r4 + u], q4[u], acc);
                 }
             }
-            acc += __shfl_xor(acc, 1, 64);
-            acc += __shfl_xor(acc, 2, 64);
+            // the quad's sum, by data-parallel-primitive moves (no trip through LDS)
+            acc += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, acc), 0xB1, 0xF, 0xF, true));  // lane ^ 1
+            acc += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, acc), 0x4E, 0xF, 0xF, true));  // lane ^ 2
             if (qd == 0) os[tt * dv_pad + j] = acc;
         }
         __syncthreads();
@@ -100,10 +163,12 @@ __global__ __launch_bounds__(1024) void gated_linear_scan_kernel(
                 ss += o * o;
             }
             ss = wave_sum(ss);
-            const float rinv = out_scale / sqrtf(ss / (float)dv + eps);
-            T* orow = out + (int64_t)(t0 + base + tt) * ld_out + (int64_t)h * dv;
-            for (int c = lane; c < dv; c += 64) orow[c] = (T)(os[tt * dv_pad + c] * rinv * gain[c]);
+            const float rinv = a.out_scale / sqrtf(ss / (float)dv + a.eps);
+            T* orow = out + (int64_t)(t0 + base + tt) * a.ld_out + (int64_t)h * dv;
+            for (int c = lane; c < dv; c += 64) orow[c] = (T)(os[tt * dv_pad + c] * rinv * a.gain[c]);
         }
+        if (n_next > 0) commit(n_next, qs + (buf ^ 1) * ts * ROW, fs + (buf ^ 1) * ts * ROW, vs + (buf ^ 1) * ts * dv_pad);
+        __syncthreads();  // the outputs are out, the next stage is in
     }
 #pragma unroll
     for (int r = 0; r < RPL; ++r) {
@@ -113,31 +178,36 @@ __global__ __launch_bounds__(1024) void gated_linear_scan_kernel(
 }
 
 template <typename T, int RPL>
-void launch_scan(const void* proj, int64_t ld, int64_t q_col0, int64_t f_col0, int64_t v_col0, const float* f_bias, const float* lower,
-                 const float* gain, float* state, const int32_t* state_slots, const int32_t* cu_q, const int32_t* positions, void* out,
-                 int64_t ld_out, float out_scale, int64_t B, int H, int dk, int dv, float eps, int q_act, hipStream_t st) {
-    const int dv_pad = (dv + 15) / 16 * 16;
-    const size_t lds = ((size_t)2 * TS * 4 * (RPL + SEG_PAD) + (size_t)2 * TS * dv_pad) * sizeof(float);
+void launch_scan(ScanArgs a, int64_t B, int64_t max_q_len, hipStream_t st) {
+    a.dv_pad = (a.dv + 15) / 16 * 16;
+    const int threads = 4 * a.dv_pad;
+    // tokens per stage: a power of two up to 32 that a thread's registers can prefetch, that 140 KiB of LDS hold (two input
+    // buffers and the outputs), and no more than the longest run needs
+    auto bytes = [&](int ts) { return ((size_t)4 * ts * 4 * (RPL + SEG_PAD) + (size_t)3 * ts * a.dv_pad) * sizeof(float); };
+    int ts = 32;
+    while (ts > 1 && (bytes(ts) > 140 * 1024 || ts >= 2 * max_q_len || ts * a.dk > PFQ * threads || ts * a.dv > PFV * threads)) ts >>= 1;
+    a.ts = ts;
+    const size_t lds = bytes(ts);
+    // wide key heads keep many rows per lane: narrow workgroups may use the registers that wide ones cannot
+    if constexpr (RPL >= 16)
+        if (threads <= 512) {
+            if (lds > 48 * 1024)
+                (void)hipFuncSetAttribute((const void*)gated_linear_scan_kernel<T, RPL, 512>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            hipLaunchKernelGGL((gated_linear_scan_kernel<T, RPL, 512>), dim3((unsigned)B, (unsigned)a.H), dim3(threads), lds, st, a);
+            return;
+        }
     if (lds > 48 * 1024)
-        (void)hipFuncSetAttribute((const void*)gated_linear_scan_kernel<T, RPL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL((gated_linear_scan_kernel<T, RPL>), dim3((unsigned)B, (unsigned)H), dim3(4 * dv_pad), lds, st, (const T*)proj, ld,
-                       q_col0, f_col0, v_col0, f_bias, lower, gain, state, state_slots, cu_q, positions, (T*)out, ld_out, out_scale, H, dk,
-                       dv, dv_pad, eps, q_act);
+        (void)hipFuncSetAttribute((const void*)gated_linear_scan_kernel<T, RPL, 1024>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL((gated_linear_scan_kernel<T, RPL, 1024>), dim3((unsigned)B, (unsigned)a.H), dim3(threads), lds, st, a);
 }
 
 template <typename T>
-void launch_scan_rows(int dk, const void* proj, int64_t ld, int64_t q_col0, int64_t f_col0, int64_t v_col0, const float* f_bias,
-                      const float* lower, const float* gain, float* state, const int32_t* state_slots, const int32_t* cu_q,
-                      const int32_t* positions, void* out, int64_t ld_out, float out_scale, int64_t B, int H, int dv, float eps, int q_act,
-                      hipStream_t st) {
-#define TGIS_SCAN(RPL) \
-    launch_scan<T, RPL>(proj, ld, q_col0, f_col0, v_col0, f_bias, lower, gain, state, state_slots, cu_q, positions, out, ld_out, out_scale, B, H, dk, dv, eps, q_act, st)
-    if (dk <= 16) TGIS_SCAN(4);
-    else if (dk <= 32) TGIS_SCAN(8);
-    else if (dk <= 64) TGIS_SCAN(16);
-    else if (dk <= 128) TGIS_SCAN(32);
-    else TGIS_SCAN(64);
-#undef TGIS_SCAN
+void launch_scan_rows(const ScanArgs& a, int64_t B, int64_t max_q_len, hipStream_t st) {
+    if (a.dk <= 16) launch_scan<T, 4>(a, B, max_q_len, st);
+    else if (a.dk <= 32) launch_scan<T, 8>(a, B, max_q_len, st);
+    else if (a.dk <= 64) launch_scan<T, 16>(a, B, max_q_len, st);
+    else if (a.dk <= 128) launch_scan<T, 32>(a, B, max_q_len, st);
+    else launch_scan<T, 64>(a, B, max_q_len, st);
 }
 
 }  // namespace
@@ -145,22 +215,21 @@ void launch_scan_rows(int dk, const void* proj, int64_t ld, int64_t q_col0, int6
 extern "C" int tgis_gated_linear_scan(const void* proj, int64_t ld, int64_t q_col0, int64_t f_col0, int64_t v_col0, const float* f_bias,
                                       const float* lower, const float* gain, float* state, const int32_t* state_slots,
                                       const int32_t* cu_seqlens_q, const int32_t* positions, void* out, int64_t ld_out, float out_scale,
-                                      int64_t B, int H, int dk, int dv, float eps, int q_act, int dtype, void* stream) {
+                                      int64_t B, int64_t max_q_len, int H, int dk, int dv, float eps, int q_act, int dtype, void* stream) {
     TGIS_CHECK_ARG(proj && gain && state && state_slots && cu_seqlens_q && positions && out, "tgis_gated_linear_scan: null tensor");
     TGIS_CHECK_ARG(H >= 1 && H <= 65535 && dk >= 1 && dk <= 256 && dv >= 1 && dv <= 256, "tgis_gated_linear_scan: heads of up to 256 x 256 (got %d x %d)", dk, dv);
     TGIS_CHECK_ARG(q_col0 >= 0 && f_col0 >= 0 && v_col0 >= 0 && ld >= q_col0 + (int64_t)H * dk && ld >= f_col0 + (int64_t)H * dk &&
-                       ld >= v_col0 + (int64_t)H * dv && ld_out >= (int64_t)H * dv,
+                       ld >= v_col0 + (int64_t)H * dv && ld_out >= (int64_t)H * dv && max_q_len >= 1,
                    "tgis_gated_linear_scan: bad strides");
     TGIS_CHECK_ARG(dtype == TGIS_F16 || dtype == TGIS_BF16 || dtype == TGIS_F32, "tgis_gated_linear_scan: bad dtype");
     if (B == 0) return TGIS_OK;
     hipStream_t st = (hipStream_t)stream;
     TgisTimedScope timed(TGIS_OP_SCAN, st);
-    if (dtype == TGIS_F16)
-        launch_scan_rows<f16>(dk, proj, ld, q_col0, f_col0, v_col0, f_bias, lower, gain, state, state_slots, cu_seqlens_q, positions, out, ld_out, out_scale, B, H, dv, eps, q_act, st);
-    else if (dtype == TGIS_BF16)
-        launch_scan_rows<bf16>(dk, proj, ld, q_col0, f_col0, v_col0, f_bias, lower, gain, state, state_slots, cu_seqlens_q, positions, out, ld_out, out_scale, B, H, dv, eps, q_act, st);
-    else
-        launch_scan_rows<float>(dk, proj, ld, q_col0, f_col0, v_col0, f_bias, lower, gain, state, state_slots, cu_seqlens_q, positions, out, ld_out, out_scale, B, H, dv, eps, q_act, st);
+    const ScanArgs a{proj, ld, q_col0, f_col0, v_col0, f_bias, lower, gain, state, state_slots, cu_seqlens_q, positions, out, ld_out, out_scale,
+                     H, dk, dv, 0, 0, eps, q_act};
+    if (dtype == TGIS_F16) launch_scan_rows<f16>(a, B, max_q_len, st);
+    else if (dtype == TGIS_BF16) launch_scan_rows<bf16>(a, B, max_q_len, st);
+    else launch_scan_rows<float>(a, B, max_q_len, st);
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
 }

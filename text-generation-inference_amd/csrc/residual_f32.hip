@@ -516,6 +516,75 @@ __global__ __launch_bounds__(256) void parallel_residual_kernel(const float* x, 
     }
 }
 
+// The same for E % 4 == 0, E <= 512 * 4 * NV and 16-byte aligned operands: 512 threads, a thread owns NV groups of four
+// consecutive elements and keeps them in registers (nothing is read twice), and the entries of the depth mix are fetched four
+// at a time before they are summed — a decode-sized step is a few rows, so the launch is a chain of round trips to memory and
+// their number is what counts.
+template <typename TD, typename TY, int NV>
+__global__ __launch_bounds__(512) void parallel_residual_vec_kernel(const float* x, GatedDelta a, GatedDelta b, float* hist, int n_prev,
+                                                                    int64_t hist_stride, const float* __restrict__ coef, float* x_out,
+                                                                    const float* __restrict__ pre_w, float pre_add, TY* __restrict__ y,
+                                                                    int64_t E, float eps) {
+    __shared__ float red[16];
+    const int64_t row = blockIdx.x;
+    f32x4 v[NV], xn[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int64_t c = ((int64_t)threadIdx.x + 512 * i) * 4;
+        v[i] = f32x4{};
+        if (c < E) {
+            v[i] = Vec4<float>::ld(x + row * E + c) + gated_delta_at<TD, 4>(a, row, c);
+            if (b.delta) v[i] += gated_delta_at<TD, 4>(b, row, c);
+        }
+        xn[i] = v[i];
+    }
+    if (hist) {
+        const float* hrow = hist + row * E;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int64_t c = ((int64_t)threadIdx.x + 512 * i) * 4;
+            if (c < E) Vec4<float>::st(hist + (int64_t)n_prev * hist_stride + row * E + c, v[i]);
+            xn[i] = v[i] * coef[n_prev];
+        }
+        int j = 0;
+        for (; j + 4 <= n_prev; j += 4) {
+            f32x4 t[4][NV];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int i = 0; i < NV; ++i) {
+                    const int64_t c = ((int64_t)threadIdx.x + 512 * i) * 4;
+                    t[u][i] = c < E ? Vec4<float>::ld(hrow + (int64_t)(j + u) * hist_stride + c) : f32x4{};
+                }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int i = 0; i < NV; ++i) xn[i] += t[u][i] * coef[j + u];
+        }
+        for (; j < n_prev; ++j)
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int64_t c = ((int64_t)threadIdx.x + 512 * i) * 4;
+                if (c < E) xn[i] += Vec4<float>::ld(hrow + (int64_t)j * hist_stride + c) * coef[j];
+            }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int64_t c = ((int64_t)threadIdx.x + 512 * i) * 4;
+        if (c < E) Vec4<float>::st(x_out + row * E + c, xn[i]);
+        ss += xn[i][0] * xn[i][0] + xn[i][1] * xn[i][1] + xn[i][2] * xn[i][2] + xn[i][3] * xn[i][3];
+    }
+    if (!pre_w) return;
+    ss = block_sum(ss, red);
+    const float rinv = 1.0f / sqrtf(ss / (float)E + eps);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int64_t c = ((int64_t)threadIdx.x + 512 * i) * 4;
+        if (c < E) Vec4<TY>::st(y + row * E + c, xn[i] * rinv * (Vec4<float>::ld(pre_w + c) + pre_add));
+    }
+}
+
 template <typename TD, typename TY>
 void launch_parallel_residual(const float* x, const GatedDelta& a, const GatedDelta& b, float* hist, int n_prev, int64_t hist_stride,
                               const float* coef, float* x_out, const float* pre_w, float pre_add, void* y, int64_t rows, int64_t E,
@@ -529,9 +598,19 @@ void launch_parallel_residual(const float* x, const GatedDelta& a, const GatedDe
     };
     const bool vec = E % 4 == 0 && ok(a) && ok(b) && al(x, 16) && al(x_out, 16) && al(hist, 16) && hist_stride % 4 == 0 && al(pre_w, 16) &&
                      al(y, 4 * sizeof(TY));
-    if (vec)
+#define TGIS_PAR_VEC(NV)                                                                                                                 \
+    hipLaunchKernelGGL((parallel_residual_vec_kernel<TD, TY, NV>), dim3((unsigned)rows), dim3(512), 0, st, x, a, b, hist, n_prev, hist_stride, \
+                       coef, x_out, pre_w, pre_add, (TY*)y, E, eps)
+    if (vec && E <= 512 * 4)
+        TGIS_PAR_VEC(1);
+    else if (vec && E <= 512 * 8)
+        TGIS_PAR_VEC(2);
+    else if (vec && E <= 512 * 16)
+        TGIS_PAR_VEC(4);
+    else if (vec)
         hipLaunchKernelGGL((parallel_residual_kernel<TD, TY, 4>), dim3((unsigned)rows), dim3(256), 0, st, x, a, b, hist, n_prev, hist_stride,
                            coef, x_out, pre_w, pre_add, (TY*)y, E, eps);
+#undef TGIS_PAR_VEC
     else
         hipLaunchKernelGGL((parallel_residual_kernel<TD, TY, 1>), dim3((unsigned)rows), dim3(256), 0, st, x, a, b, hist, n_prev, hist_stride,
                            coef, x_out, pre_w, pre_add, (TY*)y, E, eps);

@@ -139,7 +139,7 @@ SIGNATURES = {
                                       _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int, _vp, _vp, _c_i64, _c_int, _c_f, _vp, _c_i64,
                                       _c_int, _c_int, _vp]),
     "tgis_gated_linear_scan": (_c_int, [_vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_i64, _c_f,
-                                        _c_i64, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int, _vp]),
+                                        _c_i64, _c_i64, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int, _vp]),
     "tgis_moe_route_ext": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _c_int, _vp, _vp, _vp, _c_i64, _c_i64, _c_int, _c_int, _c_int, _vp]),
     "tgis_parallel_residual_f32": (_c_int, [_vp, _vp, _c_i64, _c_int, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _c_int, _vp, _vp, _c_i64, _vp,
                                             _c_int, _vp, _c_int, _c_i64, _vp, _vp, _vp, _c_f, _vp, _c_int, _c_i64, _c_i64, _c_f, _vp]),
@@ -1239,7 +1239,7 @@ def attn_varlen_win(q, k_pool, v_pool, block_tables, ctx_lens, cu_seqlens_q, H: 
 
 
 def gated_linear_scan(proj, q_col0: int, f_col0: int, v_col0: int, f_bias, lower, gain, state, state_slots, cu_seqlens_q, positions,
-                      H: int, dk: int, dv: int, eps: float, q_act: bool = True, out_scale: float = 1.0, out=None):
+                      H: int, dk: int, dv: int, eps: float, q_act: bool = True, out_scale: float = 1.0, out=None, max_q_len: int = 0):
     """S <- diag(f) S + (1 - f) v^T, o = S^T q per (sequence, head) on columns of proj [T, ld]; f = lower + (1 - lower) *
     sigmoid(proj_f + f_bias); q = silu(proj_q) if q_act; out = rms_norm(o) * gain * out_scale -> [T, H dv] (or the view `out`)."""
     assert proj.dim() == 2 and proj.stride(1) == 1
@@ -1251,7 +1251,8 @@ def gated_linear_scan(proj, q_col0: int, f_col0: int, v_col0: int, f_bias, lower
     _check(load_library().tgis_gated_linear_scan(
         _ptr(proj), proj.stride(0), q_col0, f_col0, v_col0, _f32(f_bias, "f_bias"), _f32(lower, "lower"), _f32(gain, "gain"),
         _ptr(state), _i32(state_slots, "state_slots"), _i32(cu_seqlens_q, "cu_seqlens_q"), _i32(positions, "positions"), _ptr(out),
-        out.stride(0), float(out_scale), state_slots.shape[0], H, dk, dv, float(eps), int(q_act), dtype_code3(proj.dtype), _stream()),
+        out.stride(0), float(out_scale), state_slots.shape[0], int(max_q_len) if max_q_len > 0 else max(T, 1), H, dk, dv, float(eps),
+        int(q_act), dtype_code3(proj.dtype), _stream()),
         "tgis_gated_linear_scan")
     return out
 

@@ -435,7 +435,7 @@ class GatedLinearRecurrence:
     def run(self, proj: torch.Tensor, cols, position_ids, step, out: torch.Tensor, out_scale: float = 1.0):
         native.gated_linear_scan(proj, cols[0], cols[1], cols[2], self.f_bias, self.lower, self.gain, step.state.state[self.layer_id],
                                  step.state_slots, step.cu_seqlens_q, position_ids, self.H, self.dk, self.dv, self.eps, q_act=True,
-                                 out_scale=out_scale, out=out)
+                                 out_scale=out_scale, out=out, max_q_len=step.max_q_len)
 
 
 class SideBySideMixers:
