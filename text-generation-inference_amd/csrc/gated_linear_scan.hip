@@ -9,8 +9,8 @@
 // step that starts at position 0 starts from zeros whatever the slot holds.  Gates, (1 - f), the state and the read-out are
 // fp32 whatever the activation dtype T of the projections is.
 //
-// Workgroup = (sequence, head) = dv_pad x 4 threads: a quad of neighbouring lanes shares column j of S, lane q of the quad keeps
-// rows q RPL .. q RPL + RPL - 1 in registers.  Tokens go through LDS in stages of `ts`: the stage's q and f rows (activated,
+// Workgroup = (sequence, head) = dv_pad x 4 / CPL threads: a quad of neighbouring lanes shares column j of S (and, with CPL = 2,
+// column j + dv_pad / 2), lane q of the quad keeps rows q RPL .. q RPL + RPL - 1 of its columns in registers.  Tokens go through LDS in stages of `ts`: the stage's q and f rows (activated,
 // fp32, one padded segment per row group so that the four groups' 16-byte reads fall into different banks) and v rows, in two
 // buffers.  A thread asks for its share of the NEXT stage's projections before it works through the current one (per token RPL
 // updates s = f s + (1 - f) v and RPL products for the read-out; the quad adds up by two data-parallel-primitive moves), and activates and
@@ -46,7 +46,7 @@ struct ScanArgs {
     int q_act;
 };
 
-template <typename T, int RPL, int MAXT>
+template <typename T, int RPL, int CPL, int MAXT>
 __global__ __launch_bounds__(MAXT) void gated_linear_scan_kernel(ScanArgs a) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
     constexpr int SEG = RPL + SEG_PAD, ROW = 4 * SEG;
@@ -63,12 +63,16 @@ __global__ __launch_bounds__(MAXT) void gated_linear_scan_kernel(ScanArgs a) {
     const bool fresh = a.positions[t0] == 0;
     const T* proj = reinterpret_cast<const T*>(a.proj);
     float* S = a.state + ((int64_t)a.state_slots[b] * a.H + h) * (int64_t)dk * dv;
-    float s[RPL];
+    // a lane's CPL columns are dv_pad / CPL apart
+    const int jstep = dv_pad / CPL;
+    float s[CPL][RPL];
 #pragma unroll
-    for (int r = 0; r < RPL; ++r) {
-        const int i = qd * RPL + r;
-        s[r] = (!fresh && i < dk && j < dv) ? S[(int64_t)i * dv + j] : 0.f;
-    }
+    for (int c = 0; c < CPL; ++c)
+#pragma unroll
+        for (int r = 0; r < RPL; ++r) {
+            const int i = qd * RPL + r, jc = j + c * jstep;
+            s[c][r] = (!fresh && i < dk && jc < dv) ? S[(int64_t)i * dv + jc] : 0.f;
+        }
     // rows past dk and columns past dv of both buffers: f = 1, q = 0, v = 0 (their state stays zero and is never read)
     for (int e = tid; e < 2 * ts * ROW; e += nthreads) {
         qs[e] = 0.f;
@@ -138,22 +142,34 @@ __global__ __launch_bounds__(MAXT) void gated_linear_scan_kernel(ScanArgs a) {
         const float* vb = vs + buf * ts * dv_pad + j;
 #pragma unroll 1
         for (int tt = 0; tt < n; ++tt) {
-            const float vj = vb[tt * dv_pad];
-            float acc = 0.f;
+            float vj[CPL], acc[CPL];
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) {
+                vj[c] = vb[tt * dv_pad + c * jstep];
+                acc[c] = 0.f;
+            }
 #pragma unroll
             for (int r4 = 0; r4 < RPL; r4 += 4) {
                 const f32x4 f4 = *reinterpret_cast<const f32x4*>(fb + tt * ROW + r4);
                 const f32x4 q4 = *reinterpret_cast<const f32x4*>(qb + tt * ROW + r4);
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    s[r4 + u] = fmaf(f4[u], s[r4 + u], (1.f - f4[u]) * vj);
-                    acc = fmaf(s[r4 + u], q4[u], acc);
+                    const float g = 1.f - f4[u];
+#pragma unroll
+                    for (int c = 0; c < CPL; ++c) {
+                        s[c][r4 + u] = fmaf(f4[u], s[c][r4 + u], g * vj[c]);
+                        acc[c] = fmaf(s[c][r4 + u], q4[u], acc[c]);
+                    }
                 }
             }
-            // the quad's sum, by data-parallel-primitive moves (no trip through LDS)
-            acc += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, acc), 0xB1, 0xF, 0xF, true));  // lane ^ 1
-            acc += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, acc), 0x4E, 0xF, 0xF, true));  // lane ^ 2
-            if (qd == 0) os[tt * dv_pad + j] = acc;
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) {
+                // the quad's sum, by data-parallel-primitive moves (no trip through LDS)
+                float t = acc[c];
+                t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0xB1, 0xF, 0xF, true));  // lane ^ 1
+                t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0x4E, 0xF, 0xF, true));  // lane ^ 2
+                if (qd == 0) os[tt * dv_pad + j + c * jstep] = t;
+            }
         }
         __syncthreads();
         for (int tt = wave; tt < n; tt += nw) {
@@ -171,16 +187,18 @@ __global__ __launch_bounds__(MAXT) void gated_linear_scan_kernel(ScanArgs a) {
         __syncthreads();  // the outputs are out, the next stage is in
     }
 #pragma unroll
-    for (int r = 0; r < RPL; ++r) {
-        const int i = qd * RPL + r;
-        if (i < dk && j < dv) S[(int64_t)i * dv + j] = s[r];
-    }
+    for (int c = 0; c < CPL; ++c)
+#pragma unroll
+        for (int r = 0; r < RPL; ++r) {
+            const int i = qd * RPL + r, jc = j + c * jstep;
+            if (i < dk && jc < dv) S[(int64_t)i * dv + jc] = s[c][r];
+        }
 }
 
-template <typename T, int RPL>
-void launch_scan(ScanArgs a, int64_t B, int64_t max_q_len, hipStream_t st) {
-    a.dv_pad = (a.dv + 15) / 16 * 16;
-    const int threads = 4 * a.dv_pad;
+template <typename T, int RPL, int CPL, int MAXT>
+void launch_scan_as(ScanArgs a, int64_t B, int64_t max_q_len, hipStream_t st) {
+    a.dv_pad = (a.dv + 16 * CPL - 1) / (16 * CPL) * (16 * CPL);
+    const int threads = 4 * a.dv_pad / CPL;
     // tokens per stage: a power of two up to 32 that a thread's registers can prefetch, that 140 KiB of LDS hold (two input
     // buffers and the outputs), and no more than the longest run needs
     auto bytes = [&](int ts) { return ((size_t)4 * ts * 4 * (RPL + SEG_PAD) + (size_t)3 * ts * a.dv_pad) * sizeof(float); };
@@ -188,17 +206,25 @@ void launch_scan(ScanArgs a, int64_t B, int64_t max_q_len, hipStream_t st) {
     while (ts > 1 && (bytes(ts) > 140 * 1024 || ts >= 2 * max_q_len || ts * a.dk > PFQ * threads || ts * a.dv > PFV * threads)) ts >>= 1;
     a.ts = ts;
     const size_t lds = bytes(ts);
-    // wide key heads keep many rows per lane: narrow workgroups may use the registers that wide ones cannot
-    if constexpr (RPL >= 16)
-        if (threads <= 512) {
-            if (lds > 48 * 1024)
-                (void)hipFuncSetAttribute((const void*)gated_linear_scan_kernel<T, RPL, 512>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            hipLaunchKernelGGL((gated_linear_scan_kernel<T, RPL, 512>), dim3((unsigned)B, (unsigned)a.H), dim3(threads), lds, st, a);
-            return;
-        }
     if (lds > 48 * 1024)
-        (void)hipFuncSetAttribute((const void*)gated_linear_scan_kernel<T, RPL, 1024>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL((gated_linear_scan_kernel<T, RPL, 1024>), dim3((unsigned)B, (unsigned)a.H), dim3(threads), lds, st, a);
+        (void)hipFuncSetAttribute((const void*)gated_linear_scan_kernel<T, RPL, CPL, MAXT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL((gated_linear_scan_kernel<T, RPL, CPL, MAXT>), dim3((unsigned)B, (unsigned)a.H), dim3(threads), lds, st, a);
+}
+
+// The shape of the workgroup.  Long runs are a chain of dependent tokens, and what a token costs is the length of a lane's
+// own work (its rows' updates and their LDS reads): one column per lane and as many waves as the value width gives (measured
+// at dk 64 / dv 128, 4 x 1024 tokens: 0.46 ms per layer against 0.74 with two columns per lane).  A decode step is one token per
+// sequence and mostly the state's trip from and to memory: there two columns per lane (half the waves, each read of the q / f
+// rows serves two columns) measured 5 % faster, so steps of one or two tokens take that form from 64 value channels on.
+template <typename T, int RPL>
+void launch_scan(const ScanArgs& a, int64_t B, int64_t max_q_len, hipStream_t st) {
+    if constexpr (RPL <= 32) {
+        if (a.dv >= 64 && max_q_len <= 2) return launch_scan_as<T, RPL, 2, 512>(a, B, max_q_len, st);
+    }
+    if constexpr (RPL >= 16) {
+        if (4 * ((a.dv + 15) / 16 * 16) <= 512) return launch_scan_as<T, RPL, 1, 512>(a, B, max_q_len, st);
+    }
+    launch_scan_as<T, RPL, 1, 1024>(a, B, max_q_len, st);
 }
 
 template <typename T>
