@@ -512,11 +512,14 @@ int tgis_attn_varlen_win(const void* q, int64_t ldq, const void* k_pool, const v
  *   lower, f_bias [H dk] fp32 or NULL = 0);  v = proj[v_col0 + h dv ..];
  *   S <- diag(f) S + (1 - f) v^T;  o = S^T q (the new state);  out = o / sqrt(mean(o^2) + eps) * gain[dv] * out_scale.
  * state [slots][H][dk][dv] fp32 is read (zeros when the step starts at position 0) and written back.  dk, dv <= 256;
- * max_q_len: an upper bound of a sequence's run in this step (launch shaping only). */
+ * T: tokens of the step; max_q_len: an upper bound of a sequence's run in it (launch shaping only); scratch (optional): T * H * dv
+ * floats that let a long step of few sequences deal a head's value columns to several workgroups (the norm then runs as a
+ * pass of its own over the unnormed read-outs left there). */
 int tgis_gated_linear_scan(const void* proj, int64_t ld, int64_t q_col0, int64_t f_col0, int64_t v_col0, const float* f_bias,
                            const float* lower, const float* gain, float* state, const int32_t* state_slots,
                            const int32_t* cu_seqlens_q, const int32_t* positions, void* out, int64_t ld_out, float out_scale,
-                           int64_t B, int64_t max_q_len, int H, int dk, int dv, float eps, int q_act, int dtype, void* stream);
+                           int64_t B, int64_t T, int64_t max_q_len, int H, int dk, int dv, float eps, int q_act, float* scratch,
+                           int dtype, void* stream);
 /* tgis_moe_route with a bias on the router logits (router_b [E] fp32 or NULL) and, with softmax_top != 0, weights that are the
  * softmax over the chosen logits only (0: the sigmoid of each chosen logit). */
 int tgis_moe_route_ext(const void* h, int64_t ld_h, const float* router_w, const float* router_b, const float* shared_gate_w,

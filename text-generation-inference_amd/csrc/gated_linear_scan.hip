@@ -9,9 +9,9 @@
 // step that starts at position 0 starts from zeros whatever the slot holds.  Gates, (1 - f), the state and the read-out are
 // fp32 whatever the activation dtype T of the projections is.
 //
-// Workgroup = (sequence, head) = dv_pad x 4 / CPL threads: a quad of neighbouring lanes shares column j of S (and, with CPL = 2,
-// column j + dv_pad / 2), lane q of the quad keeps rows q RPL .. q RPL + RPL - 1 of its columns in registers.  Tokens go through LDS in stages of `ts`: the stage's q and f rows (activated,
-// fp32, one padded segment per row group so that the four groups' 16-byte reads fall into different banks) and v rows, in two
+// Workgroup = (sequence, head) = dv_pad x LPC / CPL threads: LPC = 4 or 8 neighbouring lanes share column j of S (and, with
+// CPL = 2, column j + dv_pad / 2), lane q of them keeps rows q RPL .. q RPL + RPL - 1 of its columns in registers.  Tokens go through LDS in stages of `ts`: the stage's q and f rows (activated,
+// fp32, one padded segment per row group so that the groups' 16-byte reads fall into different banks) and v rows, in two
 // buffers.  A thread asks for its share of the NEXT stage's projections before it works through the current one (per token RPL
 // updates s = f s + (1 - f) v and RPL products for the read-out; the quad adds up by two data-parallel-primitive moves), and activates and
 // stores them afterwards: the trip to memory is hidden behind the arithmetic.  The stage's outputs wait in LDS for the norm,
@@ -26,7 +26,13 @@ constexpr int PFQ = 2;      // (q, f) pairs and
 constexpr int PFV = 4;      // values of the next stage that a thread holds in registers: ts dk <= PFQ threads, ts dv <= PFV threads
 
 template <typename T> __device__ __forceinline__ float ldf(const T* p) { return (float)*p; }
-__device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-z)); }
+// The logistic function in fp32: with the library's exponential and an IEEE division where the model is served in fp32, with the
+// hardware's exponential and reciprocal (a few units in the last place) where the projections it is applied to were rounded to
+// two bytes.
+template <typename T> __device__ __forceinline__ float sigmoid_as(float z) {
+    if (sizeof(T) == 4) return 1.f / (1.f + expf(-z));
+    return __builtin_amdgcn_rcpf(1.f + __expf(-z));
+}
 
 struct ScanArgs {
     const void* proj;
@@ -44,19 +50,23 @@ struct ScanArgs {
     int H, dk, dv, dv_pad, ts;
     float eps;
     int q_act;
+    // with several workgroups per head (grid.z > 1) a workgroup owns dv_pad of the head's value columns and leaves its read-outs
+    // unnormed in raw [T][H dv] for head_norm_kernel (a head's norm runs over all its columns)
+    float* raw;
 };
 
-template <typename T, int RPL, int CPL, int MAXT>
+template <typename T, int RPL, int CPL, int LPC, int MAXT>
 __global__ __launch_bounds__(MAXT) void gated_linear_scan_kernel(ScanArgs a) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
-    constexpr int SEG = RPL + SEG_PAD, ROW = 4 * SEG;
+    constexpr int SEG = RPL + SEG_PAD, ROW = LPC * SEG;
     const int ts = a.ts, dk = a.dk, dv = a.dv, dv_pad = a.dv_pad;
     float* qs = smem;                        // [2][ts][ROW]
     float* fs = qs + 2 * ts * ROW;           // [2][ts][ROW]
     float* vs = fs + 2 * ts * ROW;           // [2][ts][dv_pad]
     float* os = vs + 2 * ts * dv_pad;        // [ts][dv_pad]
     const int b = blockIdx.x, h = blockIdx.y;
-    const int tid = threadIdx.x, j = tid >> 2, qd = tid & 3;
+    const int col0 = blockIdx.z * dv_pad;  // this workgroup's first value column
+    const int tid = threadIdx.x, j = tid / LPC, qd = tid % LPC;  // LPC neighbouring lanes share a column
     const int t0 = a.cu_q[b], qlen = a.cu_q[b + 1] - t0;
     if (qlen <= 0) return;
     const int nthreads = blockDim.x;
@@ -70,7 +80,7 @@ __global__ __launch_bounds__(MAXT) void gated_linear_scan_kernel(ScanArgs a) {
     for (int c = 0; c < CPL; ++c)
 #pragma unroll
         for (int r = 0; r < RPL; ++r) {
-            const int i = qd * RPL + r, jc = j + c * jstep;
+            const int i = qd * RPL + r, jc = col0 + j + c * jstep;
             s[c][r] = (!fresh && i < dk && jc < dv) ? S[(int64_t)i * dv + jc] : 0.f;
         }
     // rows past dk and columns past dv of both buffers: f = 1, q = 0, v = 0 (their state stays zero and is never read)
@@ -79,52 +89,55 @@ __global__ __launch_bounds__(MAXT) void gated_linear_scan_kernel(ScanArgs a) {
         fs[e] = 1.f;
     }
     for (int e = tid; e < 2 * ts * dv_pad; e += nthreads) vs[e] = 0.f;
+    // A thread's share of a stage is the same in every stage — elements tid + u nthreads of the stage's [token][channel] grids — so
+    // where they come from and go to is worked out once: token within the stage, offsets into the projections and the buffers,
+    // the gate's bias and lower bound.
     T qr[PFQ], fr[PFQ], vr[PFV];
+    int q_tt[PFQ], q_src[PFQ], q_dst[PFQ], v_tt[PFV], v_src[PFV];
+    float q_fb[PFQ], q_lo[PFQ];
+#pragma unroll
+    for (int u = 0; u < PFQ; ++u) {
+        const int e = tid + u * nthreads;
+        const int tt = e / dk, i = e - tt * dk;
+        q_tt[u] = tt;
+        q_src[u] = tt * (int)a.ld + h * dk + i;
+        q_dst[u] = tt * ROW + (i / RPL) * SEG + (i % RPL);
+        q_fb[u] = a.f_bias ? a.f_bias[h * dk + i] : 0.f;
+        q_lo[u] = a.lower ? a.lower[h * dk + i] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < PFV; ++u) {
+        const int e = tid + u * nthreads;
+        const int tt = e / dv_pad, c = col0 + e - tt * dv_pad;
+        v_tt[u] = c < dv ? tt : 1 << 30;  // a column past the head's width is never fetched (its buffer entry stays zero)
+        v_src[u] = tt * (int)a.ld + h * dv + c;
+    }
     // tokens [first, first + n) of the sequence: this thread's share of their projections, as they are
     auto fetch = [&](int first, int n) {
+        const T* base = proj + (int64_t)(t0 + first) * a.ld;
 #pragma unroll
-        for (int u = 0; u < PFQ; ++u) {
-            const int e = tid + u * nthreads;
-            if (e < n * dk) {
-                const int tt = e / dk, i = e - tt * dk;
-                const T* row = proj + (int64_t)(t0 + first + tt) * a.ld + (int64_t)h * dk + i;
-                qr[u] = row[a.q_col0];
-                fr[u] = row[a.f_col0];
+        for (int u = 0; u < PFQ; ++u)
+            if (q_tt[u] < n) {
+                qr[u] = base[a.q_col0 + q_src[u]];
+                fr[u] = base[a.f_col0 + q_src[u]];
             }
-        }
 #pragma unroll
-        for (int u = 0; u < PFV; ++u) {
-            const int e = tid + u * nthreads;
-            if (e < n * dv) {
-                const int tt = e / dv, c = e - tt * dv;
-                vr[u] = proj[(int64_t)(t0 + first + tt) * a.ld + a.v_col0 + (int64_t)h * dv + c];
-            }
-        }
+        for (int u = 0; u < PFV; ++u)
+            if (v_tt[u] < n) vr[u] = base[a.v_col0 + v_src[u]];
     };
     // ... activated and stored into one stage buffer
     auto commit = [&](int n, float* qb, float* fb, float* vb) {
 #pragma unroll
-        for (int u = 0; u < PFQ; ++u) {
-            const int e = tid + u * nthreads;
-            if (e < n * dk) {
-                const int tt = e / dk, i = e - tt * dk;
+        for (int u = 0; u < PFQ; ++u)
+            if (q_tt[u] < n) {
                 float qv = (float)qr[u];
-                if (a.q_act) qv = qv * sigmoid_f(qv);
-                const float z = (float)fr[u] + (a.f_bias ? a.f_bias[h * dk + i] : 0.f);
-                const float lo = a.lower ? a.lower[h * dk + i] : 0.f;
-                const int at = tt * ROW + (i / RPL) * SEG + (i % RPL);
-                qb[at] = qv;
-                fb[at] = lo + (1.f - lo) * sigmoid_f(z);
+                if (a.q_act) qv = qv * sigmoid_as<T>(qv);
+                qb[q_dst[u]] = qv;
+                fb[q_dst[u]] = q_lo[u] + (1.f - q_lo[u]) * sigmoid_as<T>((float)fr[u] + q_fb[u]);
             }
-        }
 #pragma unroll
-        for (int u = 0; u < PFV; ++u) {
-            const int e = tid + u * nthreads;
-            if (e < n * dv) {
-                const int tt = e / dv, c = e - tt * dv;
-                vb[tt * dv_pad + c] = (float)vr[u];
-            }
-        }
+        for (int u = 0; u < PFV; ++u)
+            if (v_tt[u] < n) vb[tid + u * nthreads] = (float)vr[u];
     };
     fetch(0, min(ts, qlen));
     __syncthreads();  // the buffers are filled with their neutral values
@@ -164,15 +177,22 @@ __global__ __launch_bounds__(MAXT) void gated_linear_scan_kernel(ScanArgs a) {
             }
 #pragma unroll
             for (int c = 0; c < CPL; ++c) {
-                // the quad's sum, by data-parallel-primitive moves (no trip through LDS)
+                // the sum over the column's lanes, by data-parallel-primitive moves (no trip through LDS)
                 float t = acc[c];
                 t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0xB1, 0xF, 0xF, true));  // lane ^ 1
                 t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0x4E, 0xF, 0xF, true));  // lane ^ 2
+                if (LPC == 8)  // the other quad of the eight: lane 7 - i of the half row holds its total
+                    t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0x141, 0xF, 0xF, true));
                 if (qd == 0) os[tt * dv_pad + j + c * jstep] = t;
             }
         }
         __syncthreads();
         for (int tt = wave; tt < n; tt += nw) {
+            if (a.raw) {
+                float* rrow = a.raw + ((int64_t)(t0 + base + tt) * a.H + h) * dv + col0;
+                for (int c = lane; c < dv_pad && col0 + c < dv; c += 64) rrow[c] = os[tt * dv_pad + c];
+                continue;
+            }
             float ss = 0.f;
             for (int c = lane; c < dv; c += 64) {
                 const float o = os[tt * dv_pad + c];
@@ -190,50 +210,90 @@ __global__ __launch_bounds__(MAXT) void gated_linear_scan_kernel(ScanArgs a) {
     for (int c = 0; c < CPL; ++c)
 #pragma unroll
         for (int r = 0; r < RPL; ++r) {
-            const int i = qd * RPL + r, jc = j + c * jstep;
+            const int i = qd * RPL + r, jc = col0 + j + c * jstep;
             if (i < dk && jc < dv) S[(int64_t)i * dv + jc] = s[c][r];
         }
 }
 
-template <typename T, int RPL, int CPL, int MAXT>
-void launch_scan_as(ScanArgs a, int64_t B, int64_t max_q_len, hipStream_t st) {
-    a.dv_pad = (a.dv + 16 * CPL - 1) / (16 * CPL) * (16 * CPL);
-    const int threads = 4 * a.dv_pad / CPL;
+// out[t][h][:] = raw[t][h][:] / sqrt(mean(raw[t][h]^2) + eps) * gain * out_scale: the heads' norm after a scan whose workgroups each
+// held a part of a head's columns.  grid (token, ceil(H / 4)): a wave per head.
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_kernel(const float* __restrict__ raw, const float* __restrict__ gain, T* __restrict__ out,
+                                                        int64_t ld_out, float out_scale, int H, int dv, float eps) {
+    const int64_t t = blockIdx.x;
+    const int h = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (h >= H) return;
+    const float* r = raw + (t * H + h) * dv;
+    float v[4], ss = 0.f;  // dv <= 256
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[i] = lane + 64 * i < dv ? r[lane + 64 * i] : 0.f;
+        ss += v[i] * v[i];
+    }
+    ss = wave_sum(ss);
+    const float rinv = out_scale / sqrtf(ss / (float)dv + eps);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (lane + 64 * i < dv) out[t * ld_out + (int64_t)h * dv + lane + 64 * i] = (T)(v[i] * rinv * gain[lane + 64 * i]);
+}
+
+// cols: value columns per workgroup (a multiple of 16 CPL; the head's padded width when a workgroup holds the whole head)
+template <typename T, int RPL, int CPL, int LPC, int MAXT>
+void launch_scan_as(ScanArgs a, int64_t B, int64_t max_q_len, int cols, int col_split, int64_t T_total, hipStream_t st) {
+    a.dv_pad = cols;
+    if (col_split <= 1) a.raw = nullptr;
+    const int threads = LPC * a.dv_pad / CPL;
     // tokens per stage: a power of two up to 32 that a thread's registers can prefetch, that 140 KiB of LDS hold (two input
     // buffers and the outputs), and no more than the longest run needs
-    auto bytes = [&](int ts) { return ((size_t)4 * ts * 4 * (RPL + SEG_PAD) + (size_t)3 * ts * a.dv_pad) * sizeof(float); };
+    auto bytes = [&](int ts) { return ((size_t)4 * ts * LPC * (RPL + SEG_PAD) + (size_t)3 * ts * a.dv_pad) * sizeof(float); };
     int ts = 32;
-    while (ts > 1 && (bytes(ts) > 140 * 1024 || ts >= 2 * max_q_len || ts * a.dk > PFQ * threads || ts * a.dv > PFV * threads)) ts >>= 1;
+    while (ts > 1 && (bytes(ts) > 140 * 1024 || ts >= 2 * max_q_len || ts * a.dk > PFQ * threads || ts * a.dv_pad > PFV * threads)) ts >>= 1;
     a.ts = ts;
     const size_t lds = bytes(ts);
     if (lds > 48 * 1024)
-        (void)hipFuncSetAttribute((const void*)gated_linear_scan_kernel<T, RPL, CPL, MAXT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL((gated_linear_scan_kernel<T, RPL, CPL, MAXT>), dim3((unsigned)B, (unsigned)a.H), dim3(threads), lds, st, a);
+        (void)hipFuncSetAttribute((const void*)gated_linear_scan_kernel<T, RPL, CPL, LPC, MAXT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL((gated_linear_scan_kernel<T, RPL, CPL, LPC, MAXT>), dim3((unsigned)B, (unsigned)a.H, (unsigned)std::max(col_split, 1)),
+                       dim3(threads), lds, st, a);
+    if (a.raw)
+        hipLaunchKernelGGL(head_norm_kernel<T>, dim3((unsigned)T_total, (unsigned)((a.H + 3) / 4)), dim3(256), 0, st, a.raw, a.gain, (T*)a.out,
+                           a.ld_out, a.out_scale, a.H, a.dv, a.eps);
 }
 
-// The shape of the workgroup.  Long runs are a chain of dependent tokens, and what a token costs is the length of a lane's
-// own work (its rows' updates and their LDS reads): one column per lane and as many waves as the value width gives (measured
-// at dk 64 / dv 128, 4 x 1024 tokens: 0.46 ms per layer against 0.74 with two columns per lane).  A decode step is one token per
-// sequence and mostly the state's trip from and to memory: there two columns per lane (half the waves, each read of the q / f
-// rows serves two columns) measured 5 % faster, so steps of one or two tokens take that form from 64 value channels on.
-template <typename T, int RPL>
-void launch_scan(const ScanArgs& a, int64_t B, int64_t max_q_len, hipStream_t st) {
-    if constexpr (RPL <= 32) {
-        if (a.dv >= 64 && max_q_len <= 2) return launch_scan_as<T, RPL, 2, 512>(a, B, max_q_len, st);
+// The shape of the workgroup.  Long runs are a chain of dependent tokens; what a token costs is a wave's instructions for its
+// share of the dk dv updates (four cycles each on a 16-lane SIMD) plus its share of activating the stage.  So runs of more than
+// two tokens spread a column over EIGHT lanes where the value width leaves room for it (8 dv <= 1024 threads), else over four;
+// and when the caller gave scratch memory, value heads wider than 64 are dealt to workgroups of 64 columns — columns are
+// independent until the head's norm, which then runs as a pass of its own over the unnormed read-outs.  Measured at dk 64 /
+// dv 128, 4 x 1024 tokens, per layer: 0.46 ms with four lanes per column, 0.38 with eight, 0.24 with eight and two workgroups
+// of 64 columns (0.28 with four of 32: every workgroup activates the whole head's q and f rows).  A decode step is one token
+// per sequence and mostly the state's trip from and to memory: there four lanes per column with two columns per lane (half the
+// waves, each read of the q / f rows serves two columns) measured 5 % faster, so steps of one or two tokens take that form from
+// 64 value channels on.
+// R4: rows per lane with four lanes per column (a multiple of four, >= dk / 4); eight lanes take half of that.
+template <typename T, int R4>
+void launch_scan(const ScanArgs& a, int64_t B, int64_t max_q_len, int64_t T_total, hipStream_t st) {
+    const int pad16 = (a.dv + 15) / 16 * 16;
+    if constexpr (R4 <= 32) {
+        if (a.dv >= 64 && max_q_len <= 2) return launch_scan_as<T, R4, 2, 4, 512>(a, B, max_q_len, (a.dv + 31) / 32 * 32, 1, T_total, st);
     }
-    if constexpr (RPL >= 16) {
-        if (4 * ((a.dv + 15) / 16 * 16) <= 512) return launch_scan_as<T, RPL, 1, 512>(a, B, max_q_len, st);
+    if constexpr (R4 >= 8) {
+        if (max_q_len > 2 && a.raw && a.dv > 64 && B * a.H * ((a.dv + 63) / 64) <= 512)
+            return launch_scan_as<T, R4 / 2, 1, 8, 1024>(a, B, max_q_len, 64, (a.dv + 63) / 64, T_total, st);
+        if (max_q_len > 2 && 8 * pad16 <= 1024) return launch_scan_as<T, R4 / 2, 1, 8, 1024>(a, B, max_q_len, pad16, 1, T_total, st);
     }
-    launch_scan_as<T, RPL, 1, 1024>(a, B, max_q_len, st);
+    if constexpr (R4 >= 16) {
+        if (4 * pad16 <= 512) return launch_scan_as<T, R4, 1, 4, 512>(a, B, max_q_len, pad16, 1, T_total, st);
+    }
+    launch_scan_as<T, R4, 1, 4, 1024>(a, B, max_q_len, pad16, 1, T_total, st);
 }
 
 template <typename T>
-void launch_scan_rows(const ScanArgs& a, int64_t B, int64_t max_q_len, hipStream_t st) {
-    if (a.dk <= 16) launch_scan<T, 4>(a, B, max_q_len, st);
-    else if (a.dk <= 32) launch_scan<T, 8>(a, B, max_q_len, st);
-    else if (a.dk <= 64) launch_scan<T, 16>(a, B, max_q_len, st);
-    else if (a.dk <= 128) launch_scan<T, 32>(a, B, max_q_len, st);
-    else launch_scan<T, 64>(a, B, max_q_len, st);
+void launch_scan_rows(const ScanArgs& a, int64_t B, int64_t max_q_len, int64_t T_total, hipStream_t st) {
+    if (a.dk <= 16) launch_scan<T, 4>(a, B, max_q_len, T_total, st);
+    else if (a.dk <= 32) launch_scan<T, 8>(a, B, max_q_len, T_total, st);
+    else if (a.dk <= 64) launch_scan<T, 16>(a, B, max_q_len, T_total, st);
+    else if (a.dk <= 128) launch_scan<T, 32>(a, B, max_q_len, T_total, st);
+    else launch_scan<T, 64>(a, B, max_q_len, T_total, st);
 }
 
 }  // namespace
@@ -241,21 +301,22 @@ void launch_scan_rows(const ScanArgs& a, int64_t B, int64_t max_q_len, hipStream
 extern "C" int tgis_gated_linear_scan(const void* proj, int64_t ld, int64_t q_col0, int64_t f_col0, int64_t v_col0, const float* f_bias,
                                       const float* lower, const float* gain, float* state, const int32_t* state_slots,
                                       const int32_t* cu_seqlens_q, const int32_t* positions, void* out, int64_t ld_out, float out_scale,
-                                      int64_t B, int64_t max_q_len, int H, int dk, int dv, float eps, int q_act, int dtype, void* stream) {
+                                      int64_t B, int64_t T, int64_t max_q_len, int H, int dk, int dv, float eps, int q_act, float* scratch,
+                                      int dtype, void* stream) {
     TGIS_CHECK_ARG(proj && gain && state && state_slots && cu_seqlens_q && positions && out, "tgis_gated_linear_scan: null tensor");
     TGIS_CHECK_ARG(H >= 1 && H <= 65535 && dk >= 1 && dk <= 256 && dv >= 1 && dv <= 256, "tgis_gated_linear_scan: heads of up to 256 x 256 (got %d x %d)", dk, dv);
     TGIS_CHECK_ARG(q_col0 >= 0 && f_col0 >= 0 && v_col0 >= 0 && ld >= q_col0 + (int64_t)H * dk && ld >= f_col0 + (int64_t)H * dk &&
-                       ld >= v_col0 + (int64_t)H * dv && ld_out >= (int64_t)H * dv && max_q_len >= 1,
+                       ld >= v_col0 + (int64_t)H * dv && ld_out >= (int64_t)H * dv && max_q_len >= 1 && T >= 0,
                    "tgis_gated_linear_scan: bad strides");
     TGIS_CHECK_ARG(dtype == TGIS_F16 || dtype == TGIS_BF16 || dtype == TGIS_F32, "tgis_gated_linear_scan: bad dtype");
-    if (B == 0) return TGIS_OK;
+    if (B == 0 || T == 0) return TGIS_OK;
     hipStream_t st = (hipStream_t)stream;
     TgisTimedScope timed(TGIS_OP_SCAN, st);
     const ScanArgs a{proj, ld, q_col0, f_col0, v_col0, f_bias, lower, gain, state, state_slots, cu_seqlens_q, positions, out, ld_out, out_scale,
-                     H, dk, dv, 0, 0, eps, q_act};
-    if (dtype == TGIS_F16) launch_scan_rows<f16>(a, B, max_q_len, st);
-    else if (dtype == TGIS_BF16) launch_scan_rows<bf16>(a, B, max_q_len, st);
-    else launch_scan_rows<float>(a, B, max_q_len, st);
+                     H, dk, dv, 0, 0, eps, q_act, scratch};
+    if (dtype == TGIS_F16) launch_scan_rows<f16>(a, B, max_q_len, T, st);
+    else if (dtype == TGIS_BF16) launch_scan_rows<bf16>(a, B, max_q_len, T, st);
+    else launch_scan_rows<float>(a, B, max_q_len, T, st);
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
 }

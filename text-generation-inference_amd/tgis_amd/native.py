@@ -139,7 +139,7 @@ SIGNATURES = {
                                       _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int, _vp, _vp, _c_i64, _c_int, _c_f, _vp, _c_i64,
                                       _c_int, _c_int, _vp]),
     "tgis_gated_linear_scan": (_c_int, [_vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _c_i64, _c_f,
-                                        _c_i64, _c_i64, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int, _vp]),
+                                        _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_int, _c_f, _c_int, _vp, _c_int, _vp]),
     "tgis_moe_route_ext": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _c_int, _vp, _vp, _vp, _c_i64, _c_i64, _c_int, _c_int, _c_int, _vp]),
     "tgis_parallel_residual_f32": (_c_int, [_vp, _vp, _c_i64, _c_int, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _c_int, _vp, _vp, _c_i64, _vp,
                                             _c_int, _vp, _c_int, _c_i64, _vp, _vp, _vp, _c_f, _vp, _c_int, _c_i64, _c_i64, _c_f, _vp]),
@@ -1248,11 +1248,14 @@ def gated_linear_scan(proj, q_col0: int, f_col0: int, v_col0: int, f_bias, lower
         out = torch.empty((T, H * dv), dtype=proj.dtype, device=proj.device)
     assert out.shape == (T, H * dv) and out.stride(1) == 1 and out.dtype == proj.dtype
     assert state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (H, dk, dv)
+    mq = int(max_q_len) if max_q_len > 0 else max(T, 1)
+    # long steps: room for the unnormed read-outs, so that the kernel may deal a head's columns to several workgroups
+    scratch = torch.empty((T, H * dv), dtype=torch.float32, device=proj.device) if mq > 2 else None
     _check(load_library().tgis_gated_linear_scan(
         _ptr(proj), proj.stride(0), q_col0, f_col0, v_col0, _f32(f_bias, "f_bias"), _f32(lower, "lower"), _f32(gain, "gain"),
         _ptr(state), _i32(state_slots, "state_slots"), _i32(cu_seqlens_q, "cu_seqlens_q"), _i32(positions, "positions"), _ptr(out),
-        out.stride(0), float(out_scale), state_slots.shape[0], int(max_q_len) if max_q_len > 0 else max(T, 1), H, dk, dv, float(eps),
-        int(q_act), dtype_code3(proj.dtype), _stream()),
+        out.stride(0), float(out_scale), state_slots.shape[0], T, mq, H, dk, dv, float(eps), int(q_act), _ptr(scratch),
+        dtype_code3(proj.dtype), _stream()),
         "tgis_gated_linear_scan")
     return out
 
