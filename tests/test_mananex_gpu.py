@@ -511,10 +511,11 @@ def test_rotation_and_cache_write(gpu_device, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,dim,vdim", [(3, 16, 32), (2, 40, 64), (1, 3, 33), (2, 20, 12), (2, 128, 64), (1, 256, 128), (2, 64, 256)])
+@pytest.mark.parametrize("heads,dim,vdim", [(3, 16, 32), (2, 40, 64), (1, 3, 33), (2, 20, 12), (2, 128, 64), (1, 256, 128), (2, 64, 256), (3, 24, 96)])
 def test_gated_linear_recurrence_and_its_state(gpu_device, dtype, heads, dim, vdim):
     """The recurrence through a slot that held another sequence, whole and in portions down to one token; the state the slot
-    holds afterwards; the output scaled and written into a wider buffer."""
+    holds afterwards; the output scaled and written into a wider buffer.  Value heads wider than 64 are dealt to several
+    workgroups in the long steps (96: the last one holds half its columns), decode-sized steps give a lane two columns."""
     from tgis_amd import native
     from tgis_amd.utils.state_cache import RecurrentStateCache
 
