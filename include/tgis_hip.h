@@ -539,6 +539,69 @@ int tgis_parallel_residual_f32(const float* x, const void* a, int64_t ld_a, int 
                                float* hist, int n_prev, int64_t hist_stride, const float* mix, float* x_out, const float* pre_w,
                                float pre_add, void* y, int y_dtype, int64_t rows, int64_t E, float eps, void* stream);
 
+/* ---- parallel layers with per-channel sublayer scales, input convolutions, a selective scan, attention with scores mixed over
+ * heads, and the general linear-attention scan -------------------------------------------------------------------------- */
+/* tgis_rope_rows_kv_write, and every q and k head is divided by sqrt(mean(x^2) + unit_eps) after the rotation (no gain). */
+int tgis_rope_rows_unit_kv_write(void* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t v_col0, const float* inv_freq,
+                                 const int32_t* positions, const int32_t* slots, void* k_pool, void* v_pool, int64_t T, int H,
+                                 int G, int dk, int dv, int rot_dims, float unit_eps, int dtype, void* stream);
+/* Paged softmax attention ("rows" page layout) whose scaled scores are mixed over the query heads before the softmax:
+ * s'_h = sum_g mix[h][g] s_g, mix [H][H] fp32; a query at position i sees keys j <= i with i - j < window (window 0: all);
+ * out[t][h dv + c] is multiplied by sigmoid(gate[t][h dv + c]) when gate is given.  H dv <= 4096. */
+int tgis_attn_mixed_heads(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
+                          int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B, const float* mix,
+                          const void* gate, int64_t ld_gate, void* out, int64_t ld_out, int64_t max_q_len, int H, int G, int dk,
+                          int dv, float scale, int window, int dtype, void* stream);
+/* Linear attention S <- diag(a) S + k v^T, o = S^T q per (sequence, head) on columns of proj [T, ld]:
+ *   decay_mode 0: a = lower + (1 - lower) sigmoid(f + f_bias);  1: a = sigmoid(f + f_bias)^inv_tau;  2: a = head_decay[h];
+ *   k at k_col0 (k_col0 < 0: k = 1 - a);  q_act / k_act / v_act != 0: SiLU on the projection;  q times q_scale;
+ *   norm_rows 0: out = o / rms(o over the head) * gain[dv];  != 0: out = o / rms(o over all heads) * gain[H dv] (needs scratch);
+ *   gate_act 1: times sigmoid(gate[t][h dv + c]);  2: times SiLU of it.
+ * state [slots][H][dk][dv] fp32 as in tgis_gated_linear_scan; scratch: T * H * dv floats or NULL. */
+int tgis_linear_scan(const void* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t f_col0, int64_t v_col0,
+                     const float* f_bias, const float* lower, const float* head_decay, int decay_mode, float inv_tau, int q_act,
+                     int k_act, int v_act, float q_scale, const float* gain, int norm_rows, const void* gate, int64_t ld_gate,
+                     int gate_act, float* state, const int32_t* state_slots, const int32_t* cu_seqlens_q,
+                     const int32_t* positions, void* out, int64_t ld_out, float out_scale, int64_t B, int64_t T,
+                     int64_t max_q_len, int H, int dk, int dv, float eps, float* scratch, int dtype, void* stream);
+/* Causal per-channel convolution over time for ragged steps, `sets` (1 or 2) filter sets on the same input:
+ *   out_s[t][c] = act(bias_s[c] + sum_j w_s[c][j] x[t - (taps - 1 - j)][c]) (+ x[t][c] if residual);  act 1: SiLU.
+ * x [T, ld_x] fp32 (x_f32) or `dtype`; w [sets][C][taps], bias [sets][C] or NULL (fp32); out_s = out + s * set_stride elements,
+ * rows ld_out apart, `dtype`.  tail: slot s at tail + s * tail_stride floats holds [taps - 1][C], the inputs just before the
+ * step (zeros when the step starts at position 0); it is moved on to the step's end by the same launch. */
+int tgis_causal_conv(const void* x, int64_t ld_x, int x_f32, const float* w, const float* bias, int sets, float* tail,
+                     int64_t tail_stride, const int32_t* state_slots, const int32_t* cu_seqlens_q, const int32_t* positions,
+                     int64_t B, void* out, int64_t ld_out, int64_t set_stride, int64_t max_q_len, int64_t C, int taps, int act,
+                     int residual, int dtype, void* stream);
+/* Selective state-space scan per (sequence, channel c, state n), tokens in order:
+ *   d = softplus(dt[t][c] + dt_bias[c]);  S[c][n] <- exp(-d exp(A_log[c][n])) S[c][n] + d x[t][c] B[t][n];
+ *   out[t][c] = (sum_n S[c][n] C[t][n] + D[c] x[t][c]) silu(z[t][c]).
+ * x, z, out [T, >= inner] and bc [T, ld_bc] (B at b_col0, C at c_col0, N columns each) of `dtype`; dt fp32 (dt_f32) or `dtype`;
+ * state [slots][inner][N] fp32, read unless the step starts at position 0, written back.  N <= 128. */
+int tgis_selective_scan(const void* x, int64_t ld_x, const void* dt, int64_t ld_dt, int dt_f32, const float* dt_bias,
+                        const void* bc, int64_t ld_bc, int64_t b_col0, int64_t c_col0, const void* z, int64_t ld_z,
+                        const float* A_log, const float* D, float* state, const int32_t* state_slots,
+                        const int32_t* cu_seqlens_q, const int32_t* positions, void* out, int64_t ld_out, int64_t B,
+                        int64_t inner, int N, int dtype, void* stream);
+/* x_out = x_in + s1 * a + s2 * b + v  (each term optional; s1, s2, v [W] fp32; a, b [rows, ld] fp32 or `dtype`), and
+ * h = norm(x_out) * w with norm the mean-free layer norm (mean_free) or the RMS norm, eps inside the root; h fp32 (h_f32) or
+ * `dtype`; w NULL: no norm.  x_out may alias x_in. */
+int tgis_scaled_residual_norm(const float* x_in, float* x_out, const void* a, int64_t ld_a, int a_f32, const float* s1,
+                              const void* b, int64_t ld_b, int b_f32, const float* s2, const float* v, const float* w, void* h,
+                              int h_f32, int64_t rows, int64_t W, float eps, int mean_free, int dtype, void* stream);
+/* y = ca * a / rms(a) * wa + cb * b / rms(b) * wb over rows of W channels; a, b fp32 or `dtype`; y fp32. */
+int tgis_rms_pair_mean(const void* a, int64_t ld_a, int a_f32, const float* wa, float ca, const void* b, int64_t ld_b, int b_f32,
+                       const float* wb, float cb, float* y, int64_t rows, int64_t W, float eps, int dtype, void* stream);
+/* y = c1 z / rms(z) + c2 z^2 / rms(z^2) + c3 z^3 / rms(z^3) + c0 over rows of F values (powers element by element). */
+int tgis_poly_norm(const void* z, int64_t ld_z, void* y, int64_t ld_y, int64_t rows, int64_t F, float c1, float c2, float c3,
+                   float c0, float eps, int dtype, void* stream);
+/* Router with softmax scores over all experts: experts are chosen by score + correction[e] (fp32 [E] or NULL) among the
+ * keep_groups best of n_groups equal groups of neighbouring experts (a group ranks by its largest choice score; the other
+ * groups count as -inf); weights = the chosen experts' scores / (their sum + renorm_eps). */
+int tgis_moe_route_grouped(const void* h, int64_t ld_h, const float* router_w, const float* correction, int n_groups,
+                           int keep_groups, float renorm_eps, int32_t* idx, float* weight, int64_t T, int64_t W, int E, int k,
+                           int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

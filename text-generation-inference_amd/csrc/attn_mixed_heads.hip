@@ -1,0 +1,280 @@
+// Paged softmax attention whose scores are mixed over the query heads BEFORE the softmax ("talking heads"):
+//
+//     s_g(i, j) = scale * q_g(i) . k_kv(g)(j)                 raw score of head g (kv head floor(g / (H / G)))
+//     s'_h(i, j) = sum_g M[h][g] s_g(i, j)                     M [H, H] fp32
+//     p_h(i, .) = softmax over the visible j of s'_h(i, .)     j <= i, and i - j < window when window > 0
+//     o_h(i) = sum_j p_h(i, j) v_kv(h)(j)                      times sigmoid(gate[i][h dv + c]) when a gate is given
+//
+// A weight of head h needs the raw scores of ALL heads for its (query, key) pair, so a workgroup owns every head of a tile of
+// QT consecutive query tokens of one sequence and walks the pages the tile can see (the window's, not the context's).  Per page
+// of 32 keys: the raw scores [H][QT][32] (a thread per (head, key), the tile's queries from LDS, the key row from the page, fp32
+// sums), the mix (a thread per (head, key) again, M's row against the column of raw scores in LDS), an online softmax per
+// (head, query) over the half wave that holds its 32 keys, and the products with the values (a thread per (head, value channel):
+// the page's value rows are channel-major, 32 tokens contiguous).  Scores, weights, statistics and sums are fp32 whatever the
+// cache dtype T is.  The same kernel serves prompt portions (QT up to 8) and decode steps (QT = 1).
+//
+// Cache pages: the "rows" layout of tgis_attn_varlen — k_pool[page][kv head][token][dk], v_pool[page][kv head][dv][token].
+#include <algorithm>
+#include "common.h"
+
+namespace {
+
+constexpr int PAGE = TGIS_KV_PAGE_TOKENS;
+constexpr int THREADS = 256;
+
+struct MixArgs {
+    const void* q;
+    int64_t ldq;
+    const void* k_pool;
+    const void* v_pool;
+    const int32_t* bt;
+    int64_t bt_ld;
+    const int32_t* ctx_lens;
+    const int32_t* cu_q;
+    const float* mix;  // [H][H]
+    const void* gate;
+    int64_t ld_gate;
+    void* out;
+    int64_t ld_out;
+    int H, G, dk, dv, window;
+    float scale;
+};
+
+template <typename T> struct Vec16;
+template <> struct Vec16<float> { static constexpr int N = 4; typedef f32x4 type; };
+template <> struct Vec16<bf16> { static constexpr int N = 8; typedef bf16x8 type; };
+template <> struct Vec16<f16> { static constexpr int N = 8; typedef f16x8 type; };
+
+// OPT: output (head, channel) pairs a thread accumulates (H dv <= OPT * THREADS)
+template <typename T, int QT, int OPT>
+__global__ __launch_bounds__(THREADS) void attn_mixed_heads_kernel(MixArgs a) {
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    const int H = a.H, G = a.G, dk = a.dk, dv = a.dv, R = H / G;
+    const int b = blockIdx.y;
+    const int t0 = a.cu_q[b], qlen = a.cu_q[b + 1] - t0;
+    const int first = blockIdx.x * QT;
+    if (first >= qlen) return;
+    const int nq = min(QT, qlen - first);
+    const int ctx = a.ctx_lens[b];
+    const int pos0 = ctx - qlen + first;  // position of the tile's first query
+    const int tid = threadIdx.x;
+    const int dkp = (dk + 3) & ~3;
+    float* qs = smem;                           // [QT][H][dkp]
+    float* raw = qs + QT * H * dkp;             // [H][QT][PAGE]
+    float* pw = raw + H * QT * PAGE;            // [H][QT][PAGE] weights of the page
+    float* fac = pw + H * QT * PAGE;            // [H][QT] what the sums so far are multiplied by
+    float* lsum = fac + H * QT;                 // [H][QT] final denominators
+    const T* q = reinterpret_cast<const T*>(a.q);
+    for (int e = tid; e < QT * H * dkp; e += THREADS) {
+        const int qi = e / (H * dkp), r = e - qi * H * dkp, h = r / dkp, d = r - h * dkp;
+        qs[e] = (qi < nq && d < dk) ? (float)q[(int64_t)(t0 + first + qi) * a.ldq + (int64_t)h * dk + d] * a.scale : 0.f;
+    }
+    // a pair (head, key of the page) per thread and trip: keys are the fast index, so a half wave holds one head's 32 keys
+    const int pairs = H * PAGE;
+    const int trips = (pairs + THREADS - 1) / THREADS;
+    // running statistics of (head, query): read by the half wave that holds the head's keys, written by its first lane
+    float* mrun = lsum + H * QT;                // [H][QT]
+    float* lrun = mrun + H * QT;                // [H][QT]
+    for (int e = tid; e < H * QT; e += THREADS) {
+        mrun[e] = -INFINITY;
+        lrun[e] = 0.f;
+    }
+    float acc[OPT][QT];
+#pragma unroll
+    for (int o = 0; o < OPT; ++o)
+#pragma unroll
+        for (int qi = 0; qi < QT; ++qi) acc[o][qi] = 0.f;
+    const int lo_first = a.window > 0 ? max(pos0 - a.window + 1, 0) : 0;
+    const int last_pos = pos0 + nq - 1;
+    const T* kp = reinterpret_cast<const T*>(a.k_pool);
+    const T* vp = reinterpret_cast<const T*>(a.v_pool);
+    constexpr int VN = Vec16<T>::N;
+    typedef typename Vec16<T>::type VT;
+    const bool k_vec = dk % VN == 0;
+    __syncthreads();
+    for (int pg = lo_first / PAGE; pg <= last_pos / PAGE; ++pg) {
+        const int64_t page = a.bt[(int64_t)b * a.bt_ld + pg];
+        const int key0 = pg * PAGE;
+        // ---- raw scores ----
+        for (int tr = 0; tr < trips; ++tr) {
+            const int pr = tid + tr * THREADS;
+            if (pr >= pairs) break;
+            const int h = pr / PAGE, j = pr % PAGE;
+            const T* krow = kp + ((page * G + h / R) * PAGE + j) * (int64_t)dk;
+            float s[QT];
+#pragma unroll
+            for (int qi = 0; qi < QT; ++qi) s[qi] = 0.f;
+            if (key0 + j <= last_pos) {
+                if (k_vec) {
+                    for (int d = 0; d < dk; d += VN) {
+                        const VT kv = *reinterpret_cast<const VT*>(krow + d);
+#pragma unroll
+                        for (int qi = 0; qi < QT; ++qi) {
+                            const float* qq = qs + (qi * H + h) * dkp + d;
+#pragma unroll
+                            for (int u = 0; u < VN; u += 4) {
+                                const f32x4 q4 = *reinterpret_cast<const f32x4*>(qq + u);
+                                s[qi] = fmaf((float)kv[u], q4[0], s[qi]);
+                                s[qi] = fmaf((float)kv[u + 1], q4[1], s[qi]);
+                                s[qi] = fmaf((float)kv[u + 2], q4[2], s[qi]);
+                                s[qi] = fmaf((float)kv[u + 3], q4[3], s[qi]);
+                            }
+                        }
+                    }
+                } else {
+                    for (int d = 0; d < dk; ++d) {
+                        const float kf = (float)krow[d];
+#pragma unroll
+                        for (int qi = 0; qi < QT; ++qi) s[qi] = fmaf(kf, qs[(qi * H + h) * dkp + d], s[qi]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int qi = 0; qi < QT; ++qi) raw[(h * QT + qi) * PAGE + j] = s[qi];
+        }
+        __syncthreads();
+        // ---- mix over heads, mask, online softmax ----
+        for (int tr = 0; tr < trips; ++tr) {
+            const int pr = tid + tr * THREADS;
+            if (pr >= pairs) break;  // whole half waves leave together (pairs is a multiple of 32)
+            const int h = pr / PAGE, j = pr % PAGE;
+            float s[QT];
+#pragma unroll
+            for (int qi = 0; qi < QT; ++qi) s[qi] = 0.f;
+            for (int g = 0; g < H; ++g) {
+                const float m = a.mix[h * H + g];
+#pragma unroll
+                for (int qi = 0; qi < QT; ++qi) s[qi] = fmaf(m, raw[(g * QT + qi) * PAGE + j], s[qi]);
+            }
+            const int key = key0 + j;
+#pragma unroll
+            for (int qi = 0; qi < QT; ++qi) {
+                const int pos = pos0 + qi;
+                const bool vis = qi < nq && key <= pos && (a.window <= 0 || pos - key < a.window);
+                float v = vis ? s[qi] : -INFINITY;
+                float mx = v;
+#pragma unroll
+                for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+                const float m_old = mrun[h * QT + qi];
+                const float m_new = fmaxf(m_old, mx);
+                const float p = vis ? expf(v - m_new) : 0.f;
+                float ps = p;
+#pragma unroll
+                for (int o = 16; o > 0; o >>= 1) ps += __shfl_xor(ps, o, 64);
+                const float f = m_new == -INFINITY ? 1.f : expf(m_old - m_new);  // m_old = -inf: 0 (nothing summed yet)
+                pw[(h * QT + qi) * PAGE + j] = p;
+                if (j == 0) {
+                    fac[h * QT + qi] = f;
+                    lrun[h * QT + qi] = lrun[h * QT + qi] * f + ps;
+                    mrun[h * QT + qi] = m_new;
+                }
+            }
+        }
+        __syncthreads();
+        // ---- weights x values ----
+#pragma unroll
+        for (int o = 0; o < OPT; ++o) {
+            const int oc = tid + o * THREADS;
+            if (oc < H * dv) {
+                const int h = oc / dv, c = oc - h * dv;
+                const T* vrow = vp + ((page * G + h / R) * dv + c) * (int64_t)PAGE;
+                float vv[PAGE];
+#pragma unroll
+                for (int u = 0; u < PAGE; u += VN) {
+                    const VT v8 = *reinterpret_cast<const VT*>(vrow + u);
+#pragma unroll
+                    for (int w = 0; w < VN; ++w) vv[u + w] = (float)v8[w];
+                }
+#pragma unroll
+                for (int qi = 0; qi < QT; ++qi) {
+                    const float* pp = pw + (h * QT + qi) * PAGE;
+                    float s = 0.f;
+#pragma unroll
+                    for (int u = 0; u < PAGE; u += 4) {
+                        const f32x4 p4 = *reinterpret_cast<const f32x4*>(pp + u);
+                        // masked keys have weight zero; what a page holds is always finite (utils/kv_cache.py)
+                        s += p4[0] * vv[u] + p4[1] * vv[u + 1] + p4[2] * vv[u + 2] + p4[3] * vv[u + 3];
+                    }
+                    acc[o][qi] = acc[o][qi] * fac[h * QT + qi] + s;
+                }
+            }
+        }
+        __syncthreads();
+    }
+    T* out = reinterpret_cast<T*>(a.out);
+    const T* gate = reinterpret_cast<const T*>(a.gate);
+#pragma unroll
+    for (int o = 0; o < OPT; ++o) {
+        const int oc = tid + o * THREADS;
+        if (oc < H * dv) {
+            const int h = oc / dv;
+#pragma unroll
+            for (int qi = 0; qi < QT; ++qi)
+                if (qi < nq) {
+                    const int64_t t = t0 + first + qi;
+                    float v = acc[o][qi] / lrun[h * QT + qi];
+                    if (gate) v *= 1.f / (1.f + expf(-(float)gate[t * a.ld_gate + oc]));
+                    out[t * a.ld_out + oc] = (T)v;
+                }
+        }
+    }
+}
+
+size_t lds_bytes(int QT, int H, int dk) {
+    const int dkp = (dk + 3) & ~3;
+    return ((size_t)QT * H * dkp + (size_t)2 * H * QT * PAGE + (size_t)4 * H * QT) * sizeof(float);
+}
+
+template <typename T, int QT, int OPT>
+void launch_as(const MixArgs& a, int64_t B, int64_t max_q_len, hipStream_t st) {
+    const size_t lds = lds_bytes(QT, a.H, a.dk);
+    if (lds > 48 * 1024)
+        (void)hipFuncSetAttribute((const void*)attn_mixed_heads_kernel<T, QT, OPT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL((attn_mixed_heads_kernel<T, QT, OPT>), dim3((unsigned)cdiv64(max_q_len, QT), (unsigned)B), dim3(THREADS), lds, st, a);
+}
+
+template <typename T, int QT>
+void launch_qt(const MixArgs& a, int64_t B, int64_t max_q_len, hipStream_t st) {
+    const int per = (a.H * a.dv + THREADS - 1) / THREADS;
+    if (per <= 2) launch_as<T, QT, 2>(a, B, max_q_len, st);
+    else if (per <= 4) launch_as<T, QT, 4>(a, B, max_q_len, st);
+    else if (per <= 8) launch_as<T, QT, 8>(a, B, max_q_len, st);
+    else launch_as<T, QT, 16>(a, B, max_q_len, st);
+}
+
+template <typename T>
+void launch(const MixArgs& a, int64_t B, int64_t max_q_len, hipStream_t st) {
+    // the widest tile of queries that the step has use for, that 96 KiB of LDS hold and that keeps the accumulators in registers
+    const int per = (a.H * a.dv + THREADS - 1) / THREADS;
+    int qt = 8;
+    while (qt > 1 && (qt >= 2 * max_q_len || lds_bytes(qt, a.H, a.dk) > 96 * 1024 || per * qt > 64)) qt >>= 1;
+    if (qt == 8) launch_qt<T, 8>(a, B, max_q_len, st);
+    else if (qt == 4) launch_qt<T, 4>(a, B, max_q_len, st);
+    else if (qt == 2) launch_qt<T, 2>(a, B, max_q_len, st);
+    else launch_qt<T, 1>(a, B, max_q_len, st);
+}
+
+}  // namespace
+
+extern "C" int tgis_attn_mixed_heads(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
+                                     int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B,
+                                     const float* mix, const void* gate, int64_t ld_gate, void* out, int64_t ld_out,
+                                     int64_t max_q_len, int H, int G, int dk, int dv, float scale, int window, int dtype, void* stream) {
+    TGIS_CHECK_ARG(q && k_pool && v_pool && block_tables && ctx_lens && cu_seqlens_q && mix && out, "tgis_attn_mixed_heads: null tensor");
+    TGIS_CHECK_ARG(H >= 1 && G >= 1 && H % G == 0 && dk >= 1 && dv >= 1 && ldq >= (int64_t)H * dk && ld_out >= (int64_t)H * dv &&
+                       (!gate || ld_gate >= (int64_t)H * dv) && window >= 0 && max_q_len >= 1,
+                   "tgis_attn_mixed_heads: bad geometry (H %d, G %d, dk %d, dv %d)", H, G, dk, dv);
+    TGIS_CHECK_ARG((int64_t)H * dv <= 16 * THREADS, "tgis_attn_mixed_heads: heads x value width up to %d (got %d x %d)", 16 * THREADS, H, dv);
+    TGIS_CHECK_ARG(lds_bytes(1, H, dk) <= 150 * 1024, "tgis_attn_mixed_heads: heads x key width too large for one workgroup (%d x %d)", H, dk);
+    TGIS_CHECK_ARG(dtype == TGIS_F16 || dtype == TGIS_BF16 || dtype == TGIS_F32, "tgis_attn_mixed_heads: bad dtype");
+    if (B == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    TgisTimedScope timed(TGIS_OP_ATTN, st);
+    const MixArgs a{q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, mix, gate, ld_gate, out, ld_out, H, G, dk, dv,
+                    window, scale};
+    if (dtype == TGIS_F16) launch<f16>(a, B, max_q_len, st);
+    else if (dtype == TGIS_BF16) launch<bf16>(a, B, max_q_len, st);
+    else launch<float>(a, B, max_q_len, st);
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}

@@ -915,7 +915,7 @@ __global__ __launch_bounds__(256) void rope_rows_kv_write_kernel(T* __restrict__
                                                                  int64_t v_col0, const float* __restrict__ inv_freq,
                                                                  const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
                                                                  T* __restrict__ k_pool, T* __restrict__ v_pool, int H, int G, int dk,
-                                                                 int dv, int rdims, int v_inline) {
+                                                                 int dv, int rdims, int v_inline, float unit_eps) {
     const int64_t t = blockIdx.x;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int slot = slots[t];
@@ -939,6 +939,36 @@ __global__ __launch_bounds__(256) void rope_rows_kv_write_kernel(T* __restrict__
     T* src = is_q ? row + q_col0 + (int64_t)h * dk : row + k_col0 + (int64_t)(h - H) * dk;
     T* dst = is_q ? src : k_pool + ((page * G + (h - H)) * PAGE + off) * dk;
     const float pos = (float)positions[t];
+    if (unit_eps >= 0.f) {
+        // rotated, then divided by the head's root mean square (no gain): the rotated pairs wait in registers for the sum
+        float u[2], v[2], ss = 0.f;  // dk <= 256: two pairs per lane
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const int i = lane + 64 * r, d = 2 * i;
+            u[r] = v[r] = 0.f;
+            if (d < dk) {
+                u[r] = ldf(src + d);
+                v[r] = d + 1 < dk ? ldf(src + d + 1) : 0.f;
+                if (d + 1 < rdims) {
+                    float sn, cs;
+                    sincosf(pos * inv_freq[i], &sn, &cs);
+                    const float a = u[r] * cs - v[r] * sn, b2 = v[r] * cs + u[r] * sn;
+                    u[r] = a;
+                    v[r] = b2;
+                }
+                ss += u[r] * u[r] + v[r] * v[r];
+            }
+        }
+        ss = wave_sum(ss);
+        const float rinv = 1.f / sqrtf(ss / (float)dk + unit_eps);
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const int d = 2 * (lane + 64 * r);
+            if (d < dk) dst[d] = (T)(u[r] * rinv);
+            if (d + 1 < dk) dst[d + 1] = (T)(v[r] * rinv);
+        }
+        return;
+    }
     for (int i = lane; 2 * i < dk; i += 64) {
         const int d = 2 * i;
         if (d + 1 >= dk) {  // an odd width's last channel has no partner
@@ -1223,9 +1253,9 @@ extern "C" int tgis_latent_kv_write(const void* q, int64_t ldq, void* ckv, int64
 // Interleaved-pair rotation of q (in place) and k (into its page slot) and the value write of a step, for the "rows" page
 // layout of tgis_attn_varlen.  proj [T, ld] holds q at columns q_col0 + h dk, k at k_col0 + g dk, v at v_col0 + g dv; pair
 // (2i, 2i + 1) of the first rot_dims channels of every head turns by positions[t] * inv_freq[i] (fp32 angle), the rest pass.
-extern "C" int tgis_rope_rows_kv_write(void* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t v_col0, const float* inv_freq,
-                                       const int32_t* positions, const int32_t* slots, void* k_pool, void* v_pool, int64_t T, int H,
-                                       int G, int dk, int dv, int rot_dims, int dtype, void* stream) {
+static int rope_rows_impl(void* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t v_col0, const float* inv_freq,
+                          const int32_t* positions, const int32_t* slots, void* k_pool, void* v_pool, int64_t T, int H,
+                          int G, int dk, int dv, int rot_dims, float unit_eps, int dtype, void* stream) {
     TGIS_CHECK_ARG(proj && positions && slots && k_pool && v_pool && (inv_freq || rot_dims == 0), "tgis_rope_rows_kv_write: null tensor");
     TGIS_CHECK_ARG(H >= 1 && G >= 1 && dk >= 1 && dv >= 1 && rot_dims >= 0 && rot_dims <= dk && rot_dims % 2 == 0 && q_col0 >= 0 &&
                        k_col0 >= 0 && v_col0 >= 0 && ld >= q_col0 + (int64_t)H * dk && ld >= k_col0 + (int64_t)G * dk &&
@@ -1239,13 +1269,27 @@ extern "C" int tgis_rope_rows_kv_write(void* proj, int64_t ld, int64_t q_col0, i
     const int v_blocks = v_inline ? (int)cdiv64((int64_t)G * dv, 1024) : 0;
     TGIS_ATTN_BY_DTYPE(dtype, hipLaunchKernelGGL(rope_rows_kv_write_kernel<TT>, dim3((unsigned)T, (unsigned)((H + G + 3) / 4 + v_blocks)), dim3(256),
                                                  0, st, (TT*)proj, ld, q_col0, k_col0, v_col0, inv_freq, positions, slots, (TT*)k_pool,
-                                                 (TT*)v_pool, H, G, dk, dv, rot_dims, v_inline));
+                                                 (TT*)v_pool, H, G, dk, dv, rot_dims, v_inline, unit_eps));
     if (!v_inline)
         TGIS_ATTN_BY_DTYPE(dtype, hipLaunchKernelGGL(v_write_kernel<TT>, dim3((unsigned)cdiv64(T, 32), (unsigned)cdiv64((int64_t)G * dv, 64)),
                                                      dim3(256), 0, st, (const TT*)proj, ld, v_col0, slots, (const TT*)nullptr, (int64_t)0,
                                                      (const float*)nullptr, (TT*)v_pool, T, G, dv));
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
+}
+
+extern "C" int tgis_rope_rows_kv_write(void* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t v_col0, const float* inv_freq,
+                                       const int32_t* positions, const int32_t* slots, void* k_pool, void* v_pool, int64_t T, int H,
+                                       int G, int dk, int dv, int rot_dims, int dtype, void* stream) {
+    return rope_rows_impl(proj, ld, q_col0, k_col0, v_col0, inv_freq, positions, slots, k_pool, v_pool, T, H, G, dk, dv, rot_dims, -1.f, dtype, stream);
+}
+
+// The same, and every q and k head is divided by its root mean square (sqrt(mean(x^2) + unit_eps), no gain) after the rotation.
+extern "C" int tgis_rope_rows_unit_kv_write(void* proj, int64_t ld, int64_t q_col0, int64_t k_col0, int64_t v_col0, const float* inv_freq,
+                                            const int32_t* positions, const int32_t* slots, void* k_pool, void* v_pool, int64_t T, int H,
+                                            int G, int dk, int dv, int rot_dims, float unit_eps, int dtype, void* stream) {
+    TGIS_CHECK_ARG(unit_eps >= 0.f && dk <= 256, "tgis_rope_rows_unit_kv_write: heads of up to 256 channels, eps >= 0");
+    return rope_rows_impl(proj, ld, q_col0, k_col0, v_col0, inv_freq, positions, slots, k_pool, v_pool, T, H, G, dk, dv, rot_dims, unit_eps, dtype, stream);
 }
 
 // tgis_attn_varlen with a sliding window that also keeps the first positions (window > 0: position i sees j <= i only if

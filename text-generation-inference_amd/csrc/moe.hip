@@ -25,10 +25,13 @@ template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, int64_t ld_h, const float* __restrict__ wr,
                                                         const float* __restrict__ wg, int32_t* __restrict__ idx,
                                                         float* __restrict__ weight, float* __restrict__ shared_gate, int W, int E,
-                                                        int k, const float* __restrict__ router_b, int softmax_top) {
+                                                        int k, const float* __restrict__ router_b, int softmax_top,
+                                                        const float* __restrict__ correction, int n_groups, int keep_groups,
+                                                        float renorm_eps) {
     extern __shared__ float sm[];
     float* hs = sm;          // [W]
     float* logit = sm + W;   // [E + 1]
+    float* choice = logit + E + 1;  // [E] (softmax_top 2 only)
     const int64_t t = blockIdx.x;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
     for (int c = threadIdx.x; c < W; c += blockDim.x) hs[c] = ldf(h + t * ld_h + c);
@@ -53,6 +56,56 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
     __syncthreads();
     if (threadIdx.x == 0) {
         if (wg) shared_gate[t] = 1.f / (1.f + expf(-logit[E]));
+        if (softmax_top == 2) {
+            // scores = softmax over ALL experts; experts are chosen by score + correction among the keep_groups groups of
+            // neighbours whose best choice score is largest (the others count as -inf); weights = the chosen scores / their sum
+            float top = -INFINITY, sum = 0.f;
+            for (int e = 0; e < E; ++e) top = fmaxf(top, logit[e]);
+            for (int e = 0; e < E; ++e) sum += (logit[e] = expf(logit[e] - top));
+            for (int e = 0; e < E; ++e) {
+                logit[e] /= sum;
+                choice[e] = logit[e] + (correction ? correction[e] : 0.f);
+            }
+            if (n_groups > 1 && keep_groups < n_groups) {
+                const int per = E / n_groups;
+                // a group is dropped when at least keep_groups others beat it (ties go to the lower index)
+                for (int g = 0; g < n_groups; ++g) {
+                    float best = -INFINITY;
+                    for (int e = g * per; e < (g + 1) * per; ++e) best = fmaxf(best, choice[e]);
+                    hs[g] = best;  // the row is no longer needed
+                }
+                for (int g = 0; g < n_groups; ++g) {
+                    int ahead = 0;
+                    for (int o = 0; o < n_groups; ++o) ahead += (hs[o] > hs[g] || (hs[o] == hs[g] && o < g)) ? 1 : 0;
+                    if (ahead >= keep_groups)
+                        for (int e = g * per; e < (g + 1) * per; ++e) choice[e] = -INFINITY;
+                }
+            }
+            float wsum = 0.f;
+            for (int j = 0; j < k; ++j) {
+                int best = -1;
+                float bv = -INFINITY;
+                for (int e = 0; e < E; ++e)
+                    if (choice[e] > bv) {
+                        bv = choice[e];
+                        best = e;
+                    }
+                if (best < 0) {  // fewer allowed experts than k, or NaN scores: the first index not taken yet
+                    best = 0;
+                    for (int e = E - 1; e >= 0; --e) {
+                        bool taken = false;
+                        for (int i = 0; i < j; ++i) taken |= idx[t * k + i] == e;
+                        if (!taken) best = e;
+                    }
+                }
+                idx[t * k + j] = best;
+                weight[t * k + j] = logit[best];
+                wsum += logit[best];
+                choice[best] = -INFINITY;
+            }
+            for (int j = 0; j < k; ++j) weight[t * k + j] /= (wsum + renorm_eps);
+            return;
+        }
         // k passes of selection; ties go to the lower index
         for (int j = 0; j < k; ++j) {
             int best = -1;
@@ -305,19 +358,22 @@ extern "C" int64_t tgis_moe_row_capacity(int64_t n_pairs, int64_t E) { return (n
 
 static int moe_route_impl(const void* h, int64_t ld_h, const float* router_w, const float* shared_gate_w, int32_t* idx,
                           float* weight, float* shared_gate, int64_t T, int64_t W, int E, int k, int dtype, void* stream,
-                          const float* router_b, int softmax_top) {
+                          const float* router_b, int softmax_top, const float* correction = nullptr, int n_groups = 1,
+                          int keep_groups = 1, float renorm_eps = 0.f) {
     TGIS_CHECK_ARG(h && router_w && idx && weight && (!shared_gate_w || shared_gate), "tgis_moe_route: null tensor");
+    TGIS_CHECK_ARG(n_groups >= 1 && keep_groups >= 1 && keep_groups <= n_groups && E % n_groups == 0 && n_groups <= W,
+                   "tgis_moe_route: %d experts do not form %d equal groups", E, n_groups);
     TGIS_CHECK_ARG(E >= 1 && k >= 1 && k <= E && W >= 1 && ld_h >= W && dtype3(dtype), "tgis_moe_route: bad arguments");
-    const size_t lds = ((size_t)W + E + 1) * sizeof(float);
+    const size_t lds = ((size_t)W + 2 * E + 1) * sizeof(float);
     TGIS_CHECK_ARG(lds <= 64 * 1024, "tgis_moe_route: width + experts need %ld bytes of LDS", (long)lds);
     if (T == 0) return TGIS_OK;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == TGIS_F16)
-        hipLaunchKernelGGL(moe_route_kernel<f16>, dim3((unsigned)T), dim3(256), lds, st, (const f16*)h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, (int)W, E, k, router_b, softmax_top);
+        hipLaunchKernelGGL(moe_route_kernel<f16>, dim3((unsigned)T), dim3(256), lds, st, (const f16*)h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, (int)W, E, k, router_b, softmax_top, correction, n_groups, keep_groups, renorm_eps);
     else if (dtype == TGIS_BF16)
-        hipLaunchKernelGGL(moe_route_kernel<bf16>, dim3((unsigned)T), dim3(256), lds, st, (const bf16*)h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, (int)W, E, k, router_b, softmax_top);
+        hipLaunchKernelGGL(moe_route_kernel<bf16>, dim3((unsigned)T), dim3(256), lds, st, (const bf16*)h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, (int)W, E, k, router_b, softmax_top, correction, n_groups, keep_groups, renorm_eps);
     else
-        hipLaunchKernelGGL(moe_route_kernel<float>, dim3((unsigned)T), dim3(256), lds, st, (const float*)h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, (int)W, E, k, router_b, softmax_top);
+        hipLaunchKernelGGL(moe_route_kernel<float>, dim3((unsigned)T), dim3(256), lds, st, (const float*)h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, (int)W, E, k, router_b, softmax_top, correction, n_groups, keep_groups, renorm_eps);
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
 }
@@ -333,6 +389,15 @@ extern "C" int tgis_moe_route_ext(const void* h, int64_t ld_h, const float* rout
                                   int softmax_top, int32_t* idx, float* weight, float* shared_gate, int64_t T, int64_t W, int E, int k,
                                   int dtype, void* stream) {
     return moe_route_impl(h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, T, W, E, k, dtype, stream, router_b, softmax_top ? 1 : 0);
+}
+
+// Softmax scores over all experts; choice by score + correction [E] (fp32 or NULL) among the keep_groups best of n_groups equal
+// groups of neighbouring experts (a group's rank is its largest choice score); weights = chosen scores / (their sum + renorm_eps).
+extern "C" int tgis_moe_route_grouped(const void* h, int64_t ld_h, const float* router_w, const float* correction, int n_groups,
+                                      int keep_groups, float renorm_eps, int32_t* idx, float* weight, int64_t T, int64_t W, int E, int k,
+                                      int dtype, void* stream) {
+    return moe_route_impl(h, ld_h, router_w, nullptr, idx, weight, nullptr, T, W, E, k, dtype, stream, nullptr, 2, correction, n_groups,
+                          keep_groups, renorm_eps);
 }
 
 extern "C" int tgis_moe_align(const int32_t* idx, int64_t n_pairs, int E, int32_t* sorted, int64_t capacity, int32_t* tile_expert,

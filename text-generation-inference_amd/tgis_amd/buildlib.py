@@ -20,6 +20,8 @@ FAMILY_UNITS = {
     "lenisun": ["api", "elementwise", "gemm_dense", "residual_f32", "attn_varlen", "wkv", "moe", "sampler"],
     "senadra": ["api", "elementwise", "gemm_dense", "residual_f32", "attn_varlen", "delta_rule", "sampler"],
     "mananex": ["api", "elementwise", "gemm_dense", "residual_f32", "attn_varlen", "gated_linear_scan", "moe", "sampler"],
+    "tatevik": ["api", "elementwise", "gemm_dense", "residual_f32", "norm_f32", "attn_varlen", "attn_mixed_heads", "gated_linear_scan",
+                "selective_scan", "causal_conv", "moe", "sampler"],
 }
 
 

@@ -59,6 +59,10 @@ class BaseInferenceEngine:
             from tgis_amd.models.custom_modeling.flash_mananex_modeling import MananexConfig
 
             return MananexConfig(**raw)
+        if family == "tatevik":
+            from tgis_amd.models.custom_modeling.flash_tatevik_modeling import TatevikConfig
+
+            return TatevikConfig(**raw)
         from transformers import AutoConfig
 
         return AutoConfig.from_pretrained(model_path)

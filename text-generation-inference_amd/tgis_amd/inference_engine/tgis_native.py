@@ -12,7 +12,7 @@ from tgis_amd.utils.dist import initialize_torch_distributed
 from tgis_amd.utils.hub import local_weight_files
 from tgis_amd.utils.weights import Weights
 
-FLASH_TYPES = ["llama", "gpt_bigcode", "lenisun", "senadra", "mananex"]
+FLASH_TYPES = ["llama", "gpt_bigcode", "lenisun", "senadra", "mananex", "tatevik"]
 
 
 def _barrier(group):
@@ -50,6 +50,10 @@ def model_class_for(config):
         from tgis_amd.models.custom_modeling.flash_mananex_modeling import FlashMananexForCausalLM
 
         return FlashMananexForCausalLM, None
+    if model_type == "tatevik":
+        from tgis_amd.models.custom_modeling.flash_tatevik_modeling import FlashTatevikForCausalLM
+
+        return FlashTatevikForCausalLM, None
     raise NotImplementedError(f"Flash attention currently only supported by the following model types: {FLASH_TYPES}")
 
 

@@ -17,9 +17,9 @@ from tgis_amd.models.model import Model
 # grads are never needed in a serving shard (reference models/__init__.py:28)
 torch.set_grad_enabled(False)
 
-FLASH_MODEL_TYPES = ("llama", "gpt_bigcode", "lenisun", "senadra", "mananex")
+FLASH_MODEL_TYPES = ("llama", "gpt_bigcode", "lenisun", "senadra", "mananex", "tatevik")
 # families that exist on the flash path only, with an fp32 residual stream, their own config class and bfloat16 checkpoints
-FP32_RESIDUAL_TYPES = ("lenisun", "senadra", "mananex")
+FP32_RESIDUAL_TYPES = ("lenisun", "senadra", "mananex", "tatevik")
 
 
 def config_model_type(config: dict) -> str:

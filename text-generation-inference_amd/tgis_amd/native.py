@@ -143,6 +143,22 @@ SIGNATURES = {
     "tgis_moe_route_ext": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _c_int, _vp, _vp, _vp, _c_i64, _c_i64, _c_int, _c_int, _c_int, _vp]),
     "tgis_parallel_residual_f32": (_c_int, [_vp, _vp, _c_i64, _c_int, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _c_int, _vp, _vp, _c_i64, _vp,
                                             _c_int, _vp, _c_int, _c_i64, _vp, _vp, _vp, _c_f, _vp, _c_int, _c_i64, _c_i64, _c_f, _vp]),
+    "tgis_rope_rows_unit_kv_write": (_c_int, [_vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp, _c_i64, _c_int, _c_int, _c_int,
+                                              _c_int, _c_int, _c_f, _c_int, _vp]),
+    "tgis_attn_mixed_heads": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _vp, _c_i64, _c_i64,
+                                       _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int, _vp]),
+    "tgis_linear_scan": (_c_int, [_vp, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _c_int, _c_f, _c_int, _c_int, _c_int, _c_f,
+                                  _vp, _c_int, _vp, _c_i64, _c_int, _vp, _vp, _vp, _vp, _vp, _c_i64, _c_f, _c_i64, _c_i64, _c_i64,
+                                  _c_int, _c_int, _c_int, _c_f, _vp, _c_int, _vp]),
+    "tgis_causal_conv": (_c_int, [_vp, _c_i64, _c_int, _vp, _vp, _c_int, _vp, _c_i64, _vp, _vp, _vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64,
+                                  _c_i64, _c_int, _c_int, _c_int, _c_int, _vp]),
+    "tgis_selective_scan": (_c_int, [_vp, _c_i64, _vp, _c_i64, _c_int, _vp, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _vp, _vp, _vp, _vp,
+                                     _vp, _vp, _vp, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _vp]),
+    "tgis_scaled_residual_norm": (_c_int, [_vp, _vp, _vp, _c_i64, _c_int, _vp, _vp, _c_i64, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_i64,
+                                           _c_i64, _c_f, _c_int, _c_int, _vp]),
+    "tgis_rms_pair_mean": (_c_int, [_vp, _c_i64, _c_int, _vp, _c_f, _vp, _c_i64, _c_int, _vp, _c_f, _vp, _c_i64, _c_i64, _c_f, _c_int, _vp]),
+    "tgis_poly_norm": (_c_int, [_vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_f, _c_f, _c_f, _c_f, _c_f, _c_int, _vp]),
+    "tgis_moe_route_grouped": (_c_int, [_vp, _c_i64, _vp, _vp, _c_int, _c_int, _c_f, _vp, _vp, _c_i64, _c_i64, _c_int, _c_int, _c_int, _vp]),
 }
 
 _lib = None
@@ -1298,3 +1314,150 @@ def parallel_residual_f32(x, a, gate_a, gate_bias_a, b, gate_b, gate_bias_b, act
         _f32(pre_w, "pre_w"), float(pre_add), _ptr(y), dtype_code3(y_dtype) if y is not None else F32, rows, E, float(eps), _stream()),
         "tgis_parallel_residual_f32")
     return y
+
+
+# ---- scaled parallel layers: input convolutions, selective scan, head-mixed attention, general linear scan --------------------
+def _is_f32(t: torch.Tensor) -> int:
+    return int(t.dtype == torch.float32)
+
+
+def rope_rows_unit_kv_write(proj, q_col0: int, k_col0: int, v_col0: int, inv_freq, positions, slots, k_pool, v_pool, H: int, G: int,
+                            dk: int, dv: int, rot_dims: int, unit_eps: float):
+    """rope_rows_kv_write, then every q and k head divided by sqrt(mean(x^2) + unit_eps) (q in place, k in its page)."""
+    assert proj.dim() == 2 and proj.stride(1) == 1 and k_pool.dtype == proj.dtype and v_pool.dtype == proj.dtype
+    assert positions.shape[0] == proj.shape[0] and slots.shape[0] == proj.shape[0]
+    assert rot_dims == 0 or inv_freq.shape[0] >= rot_dims // 2
+    _check(load_library().tgis_rope_rows_unit_kv_write(
+        _ptr(proj), proj.stride(0), q_col0, k_col0, v_col0, _f32(inv_freq, "inv_freq") if rot_dims else None, _i32(positions, "positions"),
+        _i32(slots, "slots"), _ptr(k_pool), _ptr(v_pool), proj.shape[0], H, G, dk, dv, rot_dims, float(unit_eps),
+        dtype_code3(proj.dtype), _stream()), "tgis_rope_rows_unit_kv_write")
+
+
+def attn_mixed_heads(q, k_pool, v_pool, block_tables, ctx_lens, cu_seqlens_q, mix, H: int, G: int, dk: int, dv: int, scale: float,
+                     window: int = 0, gate=None, out=None, max_q_len: int = 1):
+    """Softmax attention over the paged cache with the heads' scores mixed by mix [H, H] (fp32) before the softmax; q [T, H dk]
+    (a view with unit column stride), gate [T, H dv] or None -> [T, H dv]."""
+    assert q.dim() == 2 and q.stride(1) == 1 and block_tables.dim() == 2 and mix.shape == (H, H) and mix.is_contiguous()
+    T = q.shape[0]
+    assert gate is None or (gate.dtype == q.dtype and gate.stride(1) == 1 and gate.shape == (T, H * dv))
+    if out is None:
+        out = torch.empty((T, H * dv), dtype=q.dtype, device=q.device)
+    assert out.shape == (T, H * dv) and out.stride(1) == 1 and out.dtype == q.dtype
+    _check(load_library().tgis_attn_mixed_heads(
+        _ptr(q), q.stride(0), _ptr(k_pool), _ptr(v_pool), _i32(block_tables, "block_tables"), block_tables.shape[1],
+        _i32(ctx_lens, "ctx_lens"), _i32(cu_seqlens_q, "cu_seqlens_q"), ctx_lens.shape[0], _f32(mix, "mix"), _ptr(gate),
+        gate.stride(0) if gate is not None else 0, _ptr(out), out.stride(0), max(int(max_q_len), 1), H, G, dk, dv, float(scale),
+        int(window), dtype_code3(q.dtype), _stream()), "tgis_attn_mixed_heads")
+    return out
+
+
+def linear_scan(proj, q_col0: int, k_col0: int, f_col0: int, v_col0: int, state, state_slots, cu_seqlens_q, positions, H: int, dk: int,
+                dv: int, eps: float, gain, decay_mode: int = 0, f_bias=None, lower=None, head_decay=None, inv_tau: float = 1.0,
+                q_act: bool = False, k_act: bool = False, v_act: bool = False, q_scale: float = 1.0, norm_rows: bool = False, gate=None,
+                gate_act: int = 0, out_scale: float = 1.0, out=None, max_q_len: int = 0):
+    """S <- diag(a) S + k v^T, o = S^T q on columns of proj [T, ld]; see tgis_linear_scan for the forms.  -> [T, H dv]."""
+    assert proj.dim() == 2 and proj.stride(1) == 1
+    T = proj.shape[0]
+    if out is None:
+        out = torch.empty((T, H * dv), dtype=proj.dtype, device=proj.device)
+    assert out.shape == (T, H * dv) and out.stride(1) == 1 and out.dtype == proj.dtype
+    assert state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (H, dk, dv)
+    assert gain.shape[0] == (H * dv if norm_rows else dv)
+    assert gate is None or (gate.dtype == proj.dtype and gate.stride(1) == 1 and gate.shape == (T, H * dv))
+    mq = int(max_q_len) if max_q_len > 0 else max(T, 1)
+    scratch = torch.empty((T, H * dv), dtype=torch.float32, device=proj.device) if (mq > 2 or norm_rows) else None
+    _check(load_library().tgis_linear_scan(
+        _ptr(proj), proj.stride(0), q_col0, k_col0, f_col0, v_col0, _f32(f_bias, "f_bias"), _f32(lower, "lower"),
+        _f32(head_decay, "head_decay"), int(decay_mode), float(inv_tau), int(q_act), int(k_act), int(v_act), float(q_scale),
+        _f32(gain, "gain"), int(norm_rows), _ptr(gate), gate.stride(0) if gate is not None else 0, int(gate_act) if gate is not None else 0,
+        _ptr(state), _i32(state_slots, "state_slots"), _i32(cu_seqlens_q, "cu_seqlens_q"), _i32(positions, "positions"), _ptr(out),
+        out.stride(0), float(out_scale), state_slots.shape[0], T, mq, H, dk, dv, float(eps), _ptr(scratch), dtype_code3(proj.dtype),
+        _stream()), "tgis_linear_scan")
+    return out
+
+
+def causal_conv(x, w, bias, tail, state_slots, cu_seqlens_q, positions, out_dtype, act: bool = False, residual: bool = False,
+                max_q_len: int = 0) -> torch.Tensor:
+    """x [T, >= C] (fp32 or out_dtype), w [sets, C, taps] fp32, bias [sets, C] or None, tail [slots, >= (taps - 1) * C] fp32 (a view
+    whose rows are the slots) -> out [sets, T, C]; the tail is moved on to the step's end."""
+    sets, C, taps = w.shape
+    assert x.dim() == 2 and x.stride(1) == 1 and x.shape[1] >= C and w.is_contiguous() and (x.dtype == out_dtype or x.dtype == torch.float32)
+    assert tail is None or (tail.dtype == torch.float32 and tail.dim() == 2 and tail.stride(1) == 1)
+    T = x.shape[0]
+    out = torch.empty((sets, T, C), dtype=out_dtype, device=x.device)
+    _check(load_library().tgis_causal_conv(
+        _ptr(x), x.stride(0), int(x.dtype == torch.float32 and out_dtype != torch.float32), _f32(w, "w"), _f32(bias, "bias"), sets,
+        _ptr(tail), tail.stride(0) if tail is not None else 0, _i32(state_slots, "state_slots"), _i32(cu_seqlens_q, "cu_seqlens_q"),
+        _i32(positions, "positions"), state_slots.shape[0], _ptr(out), C, T * C, int(max_q_len) if max_q_len > 0 else max(T, 1), C, taps,
+        int(act), int(residual), dtype_code3(out_dtype), _stream()), "tgis_causal_conv")
+    return out
+
+
+def selective_scan(x, dt, dt_bias, bc, b_col0: int, c_col0: int, z, A_log, D, state, state_slots, cu_seqlens_q, positions, N: int):
+    """x, z [T, inner] views, dt [T, inner] (fp32 or the activation dtype), bc [T, ld] with B | C at their columns -> [T, inner]."""
+    T, inner = x.shape
+    assert all(t.stride(1) == 1 for t in (x, dt, bc, z)) and z.shape == x.shape and dt.shape == x.shape
+    assert state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (inner, N)
+    out = torch.empty((T, inner), dtype=x.dtype, device=x.device)
+    _check(load_library().tgis_selective_scan(
+        _ptr(x), x.stride(0), _ptr(dt), dt.stride(0), int(dt.dtype == torch.float32 and x.dtype != torch.float32), _f32(dt_bias, "dt_bias"),
+        _ptr(bc), bc.stride(0), b_col0, c_col0, _ptr(z), z.stride(0), _f32(A_log, "A_log"), _f32(D, "D"), _ptr(state),
+        _i32(state_slots, "state_slots"), _i32(cu_seqlens_q, "cu_seqlens_q"), _i32(positions, "positions"), _ptr(out), out.stride(0),
+        state_slots.shape[0], inner, N, dtype_code3(x.dtype), _stream()), "tgis_selective_scan")
+    return out
+
+
+def scaled_residual_norm(x_in, a, s1, b, s2, v, w, eps: float, act_dtype, x_out=None, h_f32: bool = True, mean_free: bool = True,
+                         keep_x: bool = True):
+    """x_out = x_in + s1 * a + s2 * b + v (every term optional), h = norm(x_out) * w (w None: no norm).  -> (x_out, h); x_out may be
+    x_in; keep_x False: only h is wanted."""
+    ref = x_in if x_in is not None else (a if a is not None else b)
+    T, W = ref.shape
+    if x_out is None and keep_x:
+        x_out = torch.empty((T, W), dtype=torch.float32, device=ref.device)
+    assert x_in is None or (x_in.dtype == torch.float32 and x_in.is_contiguous())
+    assert x_out is None or (x_out.dtype == torch.float32 and x_out.is_contiguous())
+    for t in (a, b):
+        assert t is None or (t.stride(1) == 1 and t.dtype in (torch.float32, act_dtype))
+    h = None
+    if w is not None:
+        h = torch.empty((T, W), dtype=torch.float32 if h_f32 else act_dtype, device=ref.device)
+    _check(load_library().tgis_scaled_residual_norm(
+        _ptr(x_in), _ptr(x_out), _ptr(a), a.stride(0) if a is not None else 0, _is_f32(a) if a is not None else 0, _f32(s1, "s1"),
+        _ptr(b), b.stride(0) if b is not None else 0, _is_f32(b) if b is not None else 0, _f32(s2, "s2"), _f32(v, "v"), _f32(w, "w"),
+        _ptr(h), int(h_f32 or act_dtype == torch.float32), T, W, float(eps), int(mean_free), dtype_code3(act_dtype), _stream()),
+        "tgis_scaled_residual_norm")
+    return x_out, h
+
+
+def rms_pair_mean(a, wa, ca: float, b, wb, cb: float, eps: float, act_dtype) -> torch.Tensor:
+    """ca * a / rms(a) * wa + cb * b / rms(b) * wb -> fp32 [T, W]."""
+    T, W = a.shape
+    assert a.stride(1) == 1 and b.stride(1) == 1 and b.shape == a.shape
+    y = torch.empty((T, W), dtype=torch.float32, device=a.device)
+    _check(load_library().tgis_rms_pair_mean(_ptr(a), a.stride(0), _is_f32(a), _f32(wa, "wa"), float(ca), _ptr(b), b.stride(0), _is_f32(b),
+                                             _f32(wb, "wb"), float(cb), _ptr(y), T, W, float(eps), dtype_code3(act_dtype), _stream()),
+           "tgis_rms_pair_mean")
+    return y
+
+
+def poly_norm(z: torch.Tensor, c1: float, c2: float, c3: float, c0: float, eps: float) -> torch.Tensor:
+    """c1 z / rms(z) + c2 z^2 / rms(z^2) + c3 z^3 / rms(z^3) + c0 over the rows of z."""
+    assert z.dim() == 2 and z.stride(1) == 1
+    y = torch.empty(z.shape, dtype=z.dtype, device=z.device)
+    _check(load_library().tgis_poly_norm(_ptr(z), z.stride(0), _ptr(y), y.stride(0), z.shape[0], z.shape[1], float(c1), float(c2),
+                                         float(c3), float(c0), float(eps), dtype_code3(z.dtype), _stream()), "tgis_poly_norm")
+    return y
+
+
+def moe_route_grouped(h, router_w, correction, k: int, n_groups: int = 1, keep_groups: int = 1, renorm_eps: float = 0.0):
+    """(idx [T, k] int32, weight [T, k] fp32): softmax scores over all experts, choice by score + correction among the best
+    groups, weights = chosen scores / (their sum + renorm_eps)."""
+    T, W = h.shape
+    E = router_w.shape[0]
+    idx = torch.empty((T, k), dtype=torch.int32, device=h.device)
+    weight = torch.empty((T, k), dtype=torch.float32, device=h.device)
+    _check(load_library().tgis_moe_route_grouped(_ptr(h), h.stride(0), _f32(router_w, "router_w"), _f32(correction, "correction"),
+                                                 int(n_groups), int(keep_groups), float(renorm_eps), _ptr(idx), _ptr(weight), T, W, E, k,
+                                                 dtype_code3(h.dtype), _stream()), "tgis_moe_route_grouped")
+    return idx, weight

@@ -23,6 +23,14 @@ argument, so that a model file only maps its config keys and tensor names onto t
                       o = S^T silu(q), per-head RMS norm; state in a RecurrentStateCache slot
   SideBySideMixers    several mixers reading the same input through ONE stacked projection, their weighted results through
                       ONE stacked output projection
+  InputConvolutions   h + conv(h): short causal per-channel convolutions in front of sublayers that read the same input
+  SelectiveScanMixer  Mamba-style selective state-space scan behind a channel convolution, gated by SiLU(z)
+  MixedHeadAttention  rotated, unit-RMS q and k; the heads' scores mixed by a matrix before the softmax; sliding window;
+                      per-channel sigmoid output gate
+  DecayedLinearAttention  S <- diag(a) S + k v^T with a per-head constant or a learned per-channel decay; per-head or
+                      whole-row norm; sigmoid or SiLU output gate
+  NormedPairMixers    two mixers on ONE stacked projection whose results are RMS-normed over the width and averaged
+  PowerNormMLP        W_down P(W_up h), P a polynomial of the unit-RMS powers z, z^2, z^3
   ActivatedMLP        W_down act(W_up h) with the xIELU activation
   TokenSideInput      a slice of a second token embedding, gated by a GELU of a projection of the residual stream itself
 
@@ -168,10 +176,17 @@ class GatedUnit:
 
 class RoutedExperts:
     def __init__(self, weights, prefix: str, experts: int, top: int, shared: bool, router_bias: bool = False,
-                 softmax_top: bool = False, weight_on_input: bool = True):
+                 softmax_top: bool = False, weight_on_input: bool = True, grouped_softmax: bool = False, groups: int = 1,
+                 keep_groups: int = 1, renorm_eps: float = 0.0):
         """softmax_top: the routing weights are the softmax over the chosen logits (else the sigmoid of each);
-        weight_on_input: the weight scales the expert's input (else its output); router_bias: `<prefix>.router.b`."""
+        weight_on_input: the weight scales the expert's input (else its output); router_bias: `<prefix>.router.b`.
+        grouped_softmax: scores are the softmax over ALL experts; experts are chosen by score + `<prefix>.correction` among the
+        `keep_groups` best of `groups` equal groups of neighbours; weights = chosen scores / (their sum + renorm_eps)."""
         self.E, self.k = experts, top
+        self.grouped_softmax, self.groups, self.keep_groups, self.renorm_eps = bool(grouped_softmax), int(groups), int(keep_groups), float(renorm_eps)
+        if grouped_softmax and (experts % self.groups or not 1 <= self.keep_groups <= self.groups):
+            raise ValueError(f"{prefix}: {experts} experts in {groups} groups, {keep_groups} kept")
+        self.correction = _f32(weights.get_tensor(f"{prefix}.correction")) if grouped_softmax and weights.has(f"{prefix}.correction") else None
         self.softmax_top, self.weight_on_input = bool(softmax_top), bool(weight_on_input)
         self.router = _f32(weights.get_tensor(f"{prefix}.router"))
         self.router_b = _f32(weights.get_tensor(f"{prefix}.router.b")) if router_bias else None
@@ -192,7 +207,11 @@ class RoutedExperts:
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         T, W = h.shape
-        idx, weight, sg = native.moe_route(h, self.router, self.shared_gate, self.k, self.router_b, self.softmax_top)
+        if self.grouped_softmax:
+            idx, weight = native.moe_route_grouped(h, self.router, self.correction, self.k, self.groups, self.keep_groups, self.renorm_eps)
+            sg = None
+        else:
+            idx, weight, sg = native.moe_route(h, self.router, self.shared_gate, self.k, self.router_b, self.softmax_top)
         sorted_, tile_expert, pos, n_tiles = native.moe_align(idx, self.E)
         cap = sorted_.shape[0]
         hp = h if self.Wp == W else torch.nn.functional.pad(h, (0, self.Wp - W))
@@ -477,6 +496,240 @@ class SideBySideMixers:
         for m, cols, c0, sc in zip(self.mixers, self.cols, self.out_cols, self.scales):
             m.run(proj, cols, position_ids, step, heads[:, c0:c0 + m.out_width], out_scale=sc)
         return self.o(heads, partial=self.defer), proj
+
+
+class InputConvolutions:
+    """out_s = h + conv_s(h) for the sublayers s that read the same normed input h: per channel,
+    conv_s(h)_t = sum_j w_s[:, j] h_(t - taps + 1 + j), zeros before the sequence's start.  The last taps - 1 inputs of a
+    sequence wait in `floats` fp32 numbers of its state slot (one tail for all sets: it is the input's)."""
+
+    def __init__(self, weights, names, width: int, taps: int):
+        self.taps, self.width = int(taps), int(width)
+        self.w = torch.stack([_f32(weights.get_tensor(n)) for n in names]).contiguous()  # [sets, width, taps]
+        if self.w.shape[1:] != (self.width, self.taps) or not 1 <= self.taps <= 16:
+            raise ValueError(f"{names[0]}: filters {tuple(self.w.shape[1:])} for width {width}, {taps} taps (1 .. 16)")
+        self.floats = (self.taps - 1) * self.width
+
+    def forward(self, h: torch.Tensor, tail: Optional[torch.Tensor], position_ids, step, dtype):
+        """h [T, width] fp32 or `dtype`; tail: the slots' [*, floats] view -> [sets, T, width] in `dtype`."""
+        return native.causal_conv(h, self.w, None, tail, step.state_slots, step.cu_seqlens_q, position_ids, dtype, residual=True,
+                                  max_q_len=step.max_q_len)
+
+    __call__ = forward
+
+
+def _stack_rows_aligned(parts, align: int = 8):
+    """Row blocks of one weight as a stacked weight whose blocks start on multiples of `align` output columns."""
+    out, cols, at = [], [], 0
+    for w in parts:
+        cols.append(at)
+        out.append(w)
+        pad = -w.shape[0] % align
+        if pad:
+            out.append(w.new_zeros((pad, w.shape[1])))
+        at += w.shape[0] + pad
+    return torch.cat(out, 0).contiguous(), cols
+
+
+class SelectiveScanMixer:
+    """[x | z] = W_in h;  x <- silu(conv(x) + b) over `taps` taps;  [dt | B | C] = W_x x;  d = softplus(W_dt dt + b_dt);
+    S[c, n] <- exp(-d_c exp(A_log[c, n])) S[c, n] + d_c x_c B_n;  y_c = sum_n S[c, n] C_n + D_c x_c;  W_o (y * silu(z)).
+    A slot holds S [inner, state] (fp32) and the convolution's last taps - 1 inputs."""
+
+    def __init__(self, weights, prefix: str, inner: int, state: int, dt_rank: int, taps: int):
+        self.inner, self.N, self.R, self.taps = int(inner), int(state), int(dt_rank), int(taps)
+        if self.N > 128:
+            raise NotImplementedError(f"{prefix}: the selective scan keeps up to 128 states per channel (got {self.N})")
+        self.in_proj = load_linear(weights, f"{prefix}.in")
+        self.conv_w = _f32(weights.get_tensor(f"{prefix}.conv")).reshape(1, self.inner, self.taps).contiguous()
+        self.conv_b = _f32(weights.get_tensor(f"{prefix}.conv.b")).reshape(1, self.inner).contiguous()
+        wx = weights.get_tensor(f"{prefix}.x")
+        R, N = self.R, self.N
+        stacked, (self.dt_col, self.b_col, self.c_col) = _stack_rows_aligned([wx[:R], wx[R:R + N], wx[R + N:R + 2 * N]])
+        self.x_proj = FastLinear(stacked, None)
+        self.dt_proj = load_linear(weights, f"{prefix}.dt")
+        self.dt_bias = _f32(weights.get_tensor(f"{prefix}.dt.b"))
+        self.A_log = _f32(weights.get_tensor(f"{prefix}.A_log"))
+        self.D = _f32(weights.get_tensor(f"{prefix}.D"))
+        self.o = load_linear(weights, f"{prefix}.o")
+        self.kv_shape = None
+        self.state_matrix = (self.inner, self.N)
+        self.memory_floats = (self.taps - 1) * self.inner
+
+    def forward(self, h: torch.Tensor, position_ids, step, state: torch.Tensor, tail: Optional[torch.Tensor]):
+        """state: the slots' [*, inner, N]; tail: the slots' [*, memory_floats] view."""
+        xz = self.in_proj(h)
+        x = native.causal_conv(xz[:, :self.inner], self.conv_w, self.conv_b, tail, step.state_slots, step.cu_seqlens_q, position_ids,
+                               h.dtype, act=True, max_q_len=step.max_q_len)[0]
+        low = self.x_proj(x)
+        dt = self.dt_proj(_view_for_gemm(low[:, self.dt_col:self.dt_col + self.R]), out_f32=True)
+        y = native.selective_scan(x, dt, self.dt_bias, low, self.b_col, self.c_col, xz[:, self.inner:], self.A_log, self.D, state,
+                                  step.state_slots, step.cu_seqlens_q, position_ids, self.N)
+        return self.o(y, out_f32=True)
+
+
+class MixedHeadAttention:
+    """GQA softmax attention: q, k, v (and the output projection) with biases; q and k rotated in interleaved pairs over their
+    first rot_dims channels, then divided by their root mean square per head (no gain); the scaled scores of the H heads are
+    mixed by `<prefix>.talk` [H, H] before the softmax; position i sees j <= i with i - j < window (0: all); the heads'
+    outputs are multiplied channel by channel by sigmoid(W_g h).  Reads columns of its owner's projection."""
+
+    def __init__(self, weights, prefix: str, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, eps: float,
+                 window: int = 0, rot_base: float = 10000.0, rot_dims: int = 0):
+        self.H, self.G, self.dk, self.dv = heads, kv_heads, dim, vdim
+        _widths_ok_for_pages(dim, vdim)
+        if heads % kv_heads or rot_dims % 2 or rot_dims > dim or heads * vdim > 4096:
+            raise ValueError(f"{prefix}: {heads} heads of {dim} / {vdim} on {kv_heads} kv heads, {rot_dims} rotated channels")
+        self.scale, self.eps, self.window, self.rot_dims = float(scale), float(eps), int(window), int(rot_dims)
+        self.has_gate = weights.has(f"{prefix}.g")
+        self.in_names = [f"{prefix}.{n}" for n in (("q", "k", "v", "g") if self.has_gate else ("q", "k", "v"))]
+        self.out_name, self.out_width = f"{prefix}.o", heads * vdim
+        self.talk = _f32(weights.get_tensor(f"{prefix}.talk")) if weights.has(f"{prefix}.talk") else \
+            torch.eye(heads, dtype=torch.float32, device=weights.device)
+        self.inv_freq = rotary_inverse_frequencies(rot_base, self.rot_dims, weights.device) if self.rot_dims else None
+        self.kv_shape = (kv_heads, dim, vdim)
+        self.state_matrix, self.memory_floats = None, 0
+
+    def run(self, proj: torch.Tensor, cols, position_ids, step, cache_id: int, state=None) -> torch.Tensor:
+        cache = step.cache
+        k_pool, v_pool = cache.k_pool(cache_id), cache.v_pool(cache_id)
+        native.rope_rows_unit_kv_write(proj, cols[0], cols[1], cols[2], self.inv_freq, position_ids, step.slots, k_pool, v_pool,
+                                       self.H, self.G, self.dk, self.dv, self.rot_dims, self.eps)
+        gate = proj[:, cols[3]:cols[3] + self.H * self.dv] if self.has_gate else None
+        return native.attn_mixed_heads(proj[:, cols[0]:cols[0] + self.H * self.dk], k_pool, v_pool, step.block_tables, step.ctx_lens,
+                                       step.cu_seqlens_q, self.talk, self.H, self.G, self.dk, self.dv, self.scale, window=self.window,
+                                       gate=gate, max_q_len=step.max_q_len)
+
+
+class DecayedLinearAttention:
+    """Per head S <- diag(a) S + k v^T, o = S^T q (the new state is read), S fp32 in a state slot.
+      decay "head":     a = one constant per head (`head_decay`)
+      decay "channel":  a = sigmoid(W_a2 W_a1 h + b)^(1 / tau) per head and key channel (a low-rank pair `.a1`, `.a2`, `.a2.b`)
+    act: SiLU on q, k and v;  q_scale: a factor on q;  norm "head": o / rms(o) * gain[dv] per head, "row": the heads of a token
+    normed together with gain [H dv];  gate "sigmoid" / "silu": times that of W_g h.  Reads columns of its owner's projection."""
+
+    def __init__(self, weights, prefix: str, heads: int, dim: int, vdim: int, eps: float, decay: str, head_decay=None,
+                 tau: float = 1.0, act: bool = False, q_scale: float = 1.0, norm: str = "head", gate: str = "sigmoid"):
+        self.H, self.dk, self.dv, self.eps = heads, dim, vdim, float(eps)
+        if dim > 256 or vdim > 256:
+            raise NotImplementedError(f"{prefix}: the linear scan serves heads of up to 256 x 256 (got {dim} x {vdim})")
+        self.channel_decay = {"head": False, "channel": True}[decay]
+        self.act, self.q_scale, self.inv_tau = bool(act), float(q_scale), 1.0 / float(tau)
+        self.norm_rows = {"head": False, "row": True}[norm]
+        self.gate_act = {"sigmoid": 1, "silu": 2}[gate]
+        names = ["q", "k", "v", "g"] + (["a1"] if self.channel_decay else [])
+        self.in_names = [f"{prefix}.{n}" for n in names]
+        self.out_name, self.out_width = f"{prefix}.o", heads * vdim
+        self.gain = _f32(weights.get_tensor(f"{prefix}.norm"))
+        if self.gain.shape[0] != (heads * vdim if self.norm_rows else vdim):
+            raise ValueError(f"{prefix}.norm: {self.gain.shape[0]} gains for a {norm} norm of {heads} x {vdim}")
+        self.head_decay = self.a2 = self.a_bias = None
+        if self.channel_decay:
+            self.rank = weights.get_shape(f"{prefix}.a1")[0]
+            self.a2 = load_linear(weights, f"{prefix}.a2")
+            self.a_bias = _f32(weights.get_tensor(f"{prefix}.a2.b"))
+        else:
+            d = torch.tensor([float(x) for x in head_decay], dtype=torch.float32)
+            if d.shape[0] != heads:
+                raise ValueError(f"{prefix}: {d.shape[0]} decays for {heads} heads")
+            self.head_decay = d.to(weights.device)
+        self.kv_shape = None
+        self.state_matrix, self.memory_floats = (heads, dim, vdim), 0
+        # columns the mixer needs behind its owner's projection (the decay's pre-activations)
+        self.extra_cols = heads * dim if self.channel_decay else 0
+
+    def run(self, proj: torch.Tensor, cols, position_ids, step, cache_id: int, state: torch.Tensor, extra_col: int = -1) -> torch.Tensor:
+        """state: the slots' [*, H, dk, dv]; extra_col: first of this mixer's extra_cols columns of proj (channel decay)."""
+        f_col = -1
+        if self.channel_decay:
+            f_col = extra_col
+            self.a2(_view_for_gemm(proj[:, cols[4]:cols[4] + self.rank]), out=proj[:, f_col:f_col + self.H * self.dk])
+        gate = proj[:, cols[3]:cols[3] + self.H * self.dv]
+        return native.linear_scan(proj, cols[0], cols[1], f_col, cols[2], state, step.state_slots, step.cu_seqlens_q, position_ids,
+                                  self.H, self.dk, self.dv, self.eps, self.gain, decay_mode=1 if self.channel_decay else 2,
+                                  f_bias=self.a_bias, head_decay=self.head_decay, inv_tau=self.inv_tau, q_act=self.act, k_act=self.act,
+                                  v_act=self.act, q_scale=self.q_scale, norm_rows=self.norm_rows, gate=gate, gate_act=self.gate_act,
+                                  max_q_len=step.max_q_len)
+
+
+class StackedInput:
+    """Everything that reads the same input as ONE GEMM (blocks on multiples of 8 columns, biases where the names have them,
+    `extra` more columns behind the blocks for what a mixer computes from them)."""
+
+    def __init__(self, weights, names, extra: int = 0):
+        self.proj, self.cols = load_stacked_blocks(weights, names, align=8)
+        self.width = self.proj.out_features
+        self.extra_col, self.extra = self.width, int(extra)
+        if any(weights.has(n + ".b") for n in names):
+            bias = torch.zeros(self.width, dtype=self.proj.weight.dtype, device=self.proj.weight.device)
+            for n, c in zip(names, self.cols):
+                if weights.has(n + ".b"):
+                    b = weights.get_tensor(n + ".b")
+                    bias[c:c + b.shape[0]] = b
+            self.proj.bias = bias
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        if not self.extra:
+            return self.proj(h)
+        assert self.proj.bias is None
+        buf = torch.empty((h.shape[0], self.width + (self.extra + 7) // 8 * 8), dtype=h.dtype, device=h.device)
+        self.proj(h, out=buf[:, :self.width])
+        return buf
+
+    __call__ = forward
+
+
+class NormedPairMixers:
+    """Two mixers that read the same input through one stacked projection; each result goes through its own output projection
+    (a bias where `<out>.b` exists) and an RMS norm over the model width with a gain of its own; y = c (N(a) wa + N(b) wb)."""
+
+    def __init__(self, weights, left, right, left_gain: str, right_gain: str, eps: float, coef: float = 0.5):
+        self.left, self.right, self.eps, self.coef = left, right, float(eps), float(coef)
+        self.stack = StackedInput(weights, left.in_names + right.in_names)
+        n = len(left.in_names)
+        self.cols = (self.stack.cols[:n], self.stack.cols[n:])
+        self.o = []
+        for m in (left, right):
+            lin = load_linear(weights, m.out_name)
+            if weights.has(m.out_name + ".b"):
+                lin.bias = weights.get_tensor(m.out_name + ".b").contiguous()
+            self.o.append(lin)
+        self.gains = (_f32(weights.get_tensor(left_gain)), _f32(weights.get_tensor(right_gain)))
+
+    def forward(self, h: torch.Tensor, position_ids, step, cache_id: int, state) -> torch.Tensor:
+        proj = self.stack(h)
+        a = self.o[0](self.left.run(proj, self.cols[0], position_ids, step, cache_id, state), out_f32=True)
+        b = self.o[1](self.right.run(proj, self.cols[1], position_ids, step, cache_id, state), out_f32=True)
+        return native.rms_pair_mean(a, self.gains[0], self.coef, b, self.gains[1], self.coef, self.eps, h.dtype)
+
+
+class SingleMixer:
+    """One column-reading mixer behind its stacked projection and in front of its output projection."""
+
+    def __init__(self, weights, mixer):
+        self.mixer = mixer
+        self.stack = StackedInput(weights, mixer.in_names, extra=getattr(mixer, "extra_cols", 0))
+        self.o = load_linear(weights, mixer.out_name)
+
+    def forward(self, h: torch.Tensor, position_ids, step, cache_id: int, state) -> torch.Tensor:
+        proj = self.stack(h)
+        return self.o(self.mixer.run(proj, self.stack.cols, position_ids, step, cache_id, state, extra_col=self.stack.extra_col), out_f32=True)
+
+
+class PowerNormMLP:
+    """W_down (c1 N(z) + c2 N(z^2) + c3 N(z^3) + c0), z = W_up h, powers element by element, N(u) = u / sqrt(mean(u^2) + eps) over a
+    token's feed-forward values; the four numbers are `<prefix>.act` = (c1, c2, c3, c0)."""
+
+    def __init__(self, weights, prefix: str, eps: float):
+        self.up = load_linear(weights, f"{prefix}.up")
+        self.down = load_linear(weights, f"{prefix}.down")
+        self.c1, self.c2, self.c3, self.c0 = weights.get_tensor(f"{prefix}.act").float().tolist()
+        self.eps = float(eps)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        return self.down(native.poly_norm(self.up(h), self.c1, self.c2, self.c3, self.c0, self.eps), out_f32=True)
+
+    __call__ = forward
 
 
 def _softplus(z: float) -> float:
