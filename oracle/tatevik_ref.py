@@ -105,31 +105,47 @@ def mixed_head_attention(h, pos, p: Dict[str, torch.Tensor], m: dict, eps: float
     k = rotate_pairs(k, pos, float(rot.get("base", 10000.0)), int(rot.get("dims", 0)))
     q, k = rms_unit(q, eps), rms_unit(k, eps)
     st["k"], st["v"] = torch.cat([st["k"], k], 0), torch.cat([st["v"], v], 0)
-    K, V = st["k"], st["v"]
-    n = K.shape[0]
-    grp = torch.arange(H) // (H // G)
-    raw = torch.einsum("thd,nhd->htn", q, K[:, grp]) * float(m["scale"])  # [H, T, n]
-    mixed = torch.einsum("hg,gtn->htn", p["talk"], raw)
-    j = torch.arange(n)[None, :]
-    i = pos[:, None]
-    ok = (j <= i)
     window = int((m.get("mask") or {}).get("size", 0))
-    if window:
-        ok = ok & (i - j < window)
-    mixed = mixed.masked_fill(~ok[None], float("-inf"))
-    w = torch.softmax(mixed, -1)
-    o = torch.einsum("htn,nhd->thd", w, V[:, grp]).reshape(T, H * dv)
+    o = attend_mixed(q, st["k"], st["v"], pos, p["talk"], float(m["scale"]), window).reshape(T, H * dv)
     o = o * torch.sigmoid(h @ p["g"].T)
     return o @ p["o"].T + p["o.b"]
 
 
-def linear_attention(q, k, v, decay, S):
+def attend_mixed(q, K, V, pos, talk, scale: float, window: int):
+    """q [T, H, dk] at positions pos; K [n, G, dk], V [n, G, dv] of positions 0 .. n - 1.  The scaled scores of the H heads are
+    mixed by talk [H, H] before the softmax over the visible keys (j <= i, and i - j < window if window).  -> [T, H, dv]."""
+    H, G, n = q.shape[1], K.shape[1], K.shape[0]
+    grp = torch.arange(H) // (H // G)
+    raw = torch.einsum("thd,nhd->htn", q, K[:, grp]) * scale  # [H, T, n]
+    mixed = torch.einsum("hg,gtn->htn", talk, raw)
+    j = torch.arange(n)[None, :]
+    i = pos[:, None]
+    ok = (j <= i)
+    if window:
+        ok = ok & (i - j < window)
+    mixed = mixed.masked_fill(~ok[None], float("-inf"))
+    w = torch.softmax(mixed, -1)
+    return torch.einsum("htn,nhd->thd", w, V[:, grp])
+
+
+# When these are lists, route() appends how far each token is from another choice of experts and linear_attention() how much of
+# a read-out's terms survive their cancellation (clear_cut_tokens uses them to draw prompts that rounding cannot tip).
+ROUTER_MARGINS: Optional[list] = None
+READOUT_CONDITION: Optional[list] = None
+
+
+def linear_attention(q, k, v, decay, S, S_abs=None):
     """S_t = diag(decay_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t per head.  q, k [T, H, dk], v [T, H, dv], decay [T, H, dk]
     (broadcastable), S [H, dk, dv].  Returns (o [T, H, dv], S)."""
     outs = []
     for t in range(q.shape[0]):
         S = decay[t][..., None] * S + k[t][..., None] * v[t][:, None, :]
-        outs.append(torch.einsum("hkv,hk->hv", S, q[t]))
+        o = torch.einsum("hkv,hk->hv", S, q[t])
+        outs.append(o)
+        if READOUT_CONDITION is not None and S_abs is not None:
+            S_abs[0] = decay[t][..., None] * S_abs[0] + k[t].abs()[..., None] * v[t].abs()[:, None, :]
+            terms = torch.einsum("hkv,hk->hv", S_abs[0], q[t].abs())
+            READOUT_CONDITION.append(float((o.norm(dim=-1) / terms.norm(dim=-1).clamp_min(1e-300)).min()))
     return torch.stack(outs), S
 
 
@@ -142,7 +158,7 @@ def fixed_decay_attention(h, p, m: dict, eps: float, st: dict):
     k = silu(h @ p["k"].T).view(T, H, dk)
     v = silu(h @ p["v"].T).view(T, H, dv)
     decay = torch.tensor(m["decay"], dtype=DT).view(1, H, 1).expand(T, H, dk)
-    o, st["S"] = linear_attention(q, k, v, decay, st["S"])
+    o, st["S"] = linear_attention(q, k, v, decay, st["S"], st.setdefault("S_abs", [torch.zeros_like(st["S"])]))
     o = rms_unit(o.reshape(T, H * dv), eps) * p["norm"] * torch.sigmoid(h @ p["g"].T)
     return o @ p["o"].T
 
@@ -163,7 +179,7 @@ def channel_decay_attention(h, p, m: dict, eps: float, st: dict):
     v = (h @ p["v"].T).view(T, H, dv)
     z = (h @ p["a1"].T) @ p["a2"].T + p["a2.b"]
     decay = torch.exp(torch.nn.functional.logsigmoid(z) / float(m["tau"])).view(T, H, dk)
-    o, st["S"] = linear_attention(q, k, v, decay, st["S"])
+    o, st["S"] = linear_attention(q, k, v, decay, st["S"], st.setdefault("S_abs", [torch.zeros_like(st["S"])]))
     o = (rms_unit(o, eps) * p["norm"]).reshape(T, H * dv) * silu(h @ p["g"].T)
     return o @ p["o"].T
 
@@ -185,9 +201,15 @@ def route(h, p, r: dict):
     count, keep = int(groups.get("count", 1)), int(groups.get("keep", groups.get("count", 1)))
     if count > 1 and keep < count:
         best = c.view(-1, count, E // count).max(-1).values
+        if ROUTER_MARGINS is not None:
+            b = best.sort(-1, descending=True).values
+            ROUTER_MARGINS.extend((b[:, keep - 1] - b[:, keep]).tolist())
         kept = best.topk(keep, -1).indices
         allow = torch.zeros_like(best, dtype=torch.bool).scatter_(1, kept, True)
         c = c.masked_fill(~allow[:, :, None].expand(-1, -1, E // count).reshape(-1, E), float("-inf"))
+    if ROUTER_MARGINS is not None and top < E:
+        b = c.sort(-1, descending=True).values
+        ROUTER_MARGINS.extend(float(x) for x in (b[:, top - 1] - b[:, top]).tolist() if x == x and x != float("inf"))
     idx = c.topk(top, -1).indices
     w = s.gather(1, idx)
     return idx, w / (w.sum(-1, keepdim=True) + 1e-20), s, c
@@ -298,3 +320,30 @@ class TatevikRef:
 
     def forward(self, tokens: List[int], trace: Optional[list] = None) -> torch.Tensor:
         return self.advance(self.new_state(), tokens, trace)
+
+
+def clear_cut_tokens(config: dict, tensors, n: int, seed: int, margin: float = 0.05, condition: float = 0.05) -> List[int]:
+    """n random tokens, each drawn again until no router of the model is within `margin` (in score) of choosing other experts
+    or groups for it and no read-out of a linear attention cancels to less than `condition` of its terms before it is normed:
+    what a reduced-precision run computes for them differs from this restatement by rounding, not by a decision or a division
+    that rounding tips."""
+    import copy
+
+    global ROUTER_MARGINS, READOUT_CONDITION
+    g = torch.Generator().manual_seed(seed)
+    ref = TatevikRef(config, tensors)
+    state, toks = ref.new_state(), []
+    try:
+        while len(toks) < n:
+            for _ in range(50):
+                t = int(torch.randint(0, config["vocab"], (1,), generator=g))
+                trial = copy.deepcopy(state)
+                ROUTER_MARGINS, READOUT_CONDITION = [], []
+                ref.advance(trial, [t])
+                if all(m >= margin for m in ROUTER_MARGINS) and all(c >= condition for c in READOUT_CONDITION):
+                    break
+            state = trial
+            toks.append(t)
+    finally:
+        ROUTER_MARGINS = READOUT_CONDITION = None
+    return toks

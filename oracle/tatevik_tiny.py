@@ -130,7 +130,7 @@ def make_tensors(config: dict, seed: int = 0, dtype=torch.bfloat16) -> Dict[str,
                     lin(f"{q}.e{e}.gate", f["expert"]["ff"], W)
                     lin(f"{q}.e{e}.up", f["expert"]["ff"], W)
                     lin(f"{q}.e{e}.down", W, f["expert"]["ff"], 2.0)
-                lin(f"{q}.router", E, W, 3.0)
+                lin(f"{q}.router", E, W, 1.5)
                 vec(f"{q}.correction", E, 0.0, 0.15)
     vec("final.norm", W, 1.0)
     lin("head", config["vocab"], W)
@@ -146,4 +146,4 @@ def standard_layers() -> List[dict]:
             pair_layer(left=attention_part(heads=4, kv_heads=4, dim=16, vdim=16, window=None, rot_dims=16),
                        right=fixed_decay_part(heads=2, dim=32, vdim=16, decay=(0.5, 0.99)), mlp=dense_mlp(ff=64)),
             scan_layer(inner=80, state=16, dt_rank=5, conv=2, mlp=moe_mlp(experts=4, top=1, ff=56, groups=1, keep=1)),
-            channel_decay_layer(heads=2, dim=40, vdim=24, tau=3.0, rank=16, mlp=moe_mlp(experts=8, top=3, ff=32, groups=4, keep=1))]
+            channel_decay_layer(heads=2, dim=40, vdim=24, tau=3.0, rank=16, mlp=moe_mlp(experts=8, top=3, ff=32, groups=4, keep=2))]
