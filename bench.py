@@ -456,6 +456,38 @@ def mananex_layers(variant, width, layers, heads, kv_heads, dim, ff):
     return out
 
 
+def tatevik_layers(variant, width, layers, heads, kv_heads, dim, ff):
+    """"tatevik_pair": every layer the two mixers side by side (head-mixed attention with a window longer than any context here,
+    so that the cache bytes equal Llama's, beside a fixed-decay linear attention of width / 256 heads of 64 x 128) + the
+    power-norm feed-forward of 3 ff / 2 (the parameters of a gated unit of ff) — like for like with Mananex "mananex_dense".
+    "tatevik": selective scan / side-by-side pair with a window of 512 / two channel-decay linear attentions in turn, every
+    second feed-forward a mixture of 8 experts of ff / 4 in 2 groups of which one is kept, top 2; input convolutions of 4 taps;
+    the middle of the stack is a loop of two passes, so that `layers` layer runs share fewer layers' weights — the design as it
+    is meant.  Returns (layers, loop, canon taps)."""
+    pair = lambda window: {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                    "mask": {"size": window}, "rot": {"base": 10000.0, "dims": dim}},
+                           "right": {"heads": max(1, width // 256), "dim": 64, "vdim": 128,
+                                     "decay": [1.0 - 2.0 ** (-3 - j % 6) for j in range(max(1, width // 256))]}}
+    if variant == "tatevik_pair":
+        return [{"type": "parallel", "mixer": pair(8192), "mlp": {"kind": "dense", "ff": 3 * ff // 2}} for _ in range(layers)], None, 0
+    span = layers // 3
+    n_weights = layers - span  # `span` layers run twice
+    out = []
+    for i in range(n_weights):
+        mlp = {"kind": "dense", "ff": 3 * ff // 2}
+        if i % 2 == 1:
+            mlp = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 8, "top": 2, "groups": {"count": 2, "keep": 1}}}
+        kind = ("mamba1", "parallel", "gla", "gla")[i % 4]
+        if kind == "mamba1":
+            mixer = {"inner": 2 * width, "state": 16, "dt_rank": width // 16, "conv": 4}
+        elif kind == "parallel":
+            mixer = pair(512)
+        else:
+            mixer = {"heads": max(1, width // 256), "dim": 64, "vdim": 128, "tau": 16.0}
+        out.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    return out, {"start": 1, "stop": 1 + span, "times": 2}, 4
+
+
 def bench_hybrid(args):
     """Prefill and decode throughput + per-kernel-class device time (HIP events, eager pass) of Lenisun variants and of
     Llama at the same size, through the same entry points (from_pb -> generate_token).  One JSON line."""
@@ -495,6 +527,15 @@ def bench_hybrid(args):
             cfg = MananexConfig(width=width, vocab=vocab, norm={"eps": 1e-5}, layers=mananex_layers(name, width, layers, heads, kv_heads, dim, ff))
             tensors = mananex_tensors(cfg, seed=1234, device=device, dtype=dtype)
             n_attn = n_scan = layers
+        elif name.startswith("tatevik"):
+            from tgis_amd.inference_engine.synthetic import tatevik_tensors
+            from tgis_amd.models.custom_modeling.flash_tatevik_modeling import TatevikConfig
+
+            lays, loop, taps = tatevik_layers(name, width, layers, heads, kv_heads, dim, ff)
+            cfg = TatevikConfig(width=width, vocab=vocab, norm={"eps": 1e-5}, layers=lays, loop=loop, canon={"taps": taps} if taps else None)
+            tensors = tatevik_tensors(cfg, seed=1234, device=device, dtype=dtype)
+            n_attn = sum(cfg.layers[i]["type"] == "parallel" for i, _ in cfg.runs)
+            n_scan = len(cfg.runs)  # every run has one: selective scan, fixed-decay or channel-decay linear attention
         elif name.startswith("senadra"):
             cfg = SenadraConfig(width=width, vocab=vocab, norm={"eps": 1e-5}, residual_mult=0.25, token_side={"dim": 64},
                                 logit_softcap=25.0, layers=senadra_layers(name, width, layers, heads, kv_heads, dim, ff))
@@ -564,7 +605,7 @@ def bench_hybrid(args):
             ctx_now = L_in + W + K + 2
             if "attention" in kern:
                 # bytes one attention launch has to read: every cached key and value of the batch once
-                keys = min(ctx_now, 512 + 4 + 32) if name == "mananex" else ctx_now  # a window, its kept positions, a page's slack
+                keys = min(ctx_now, 512 + 4 + 32) if name in ("mananex", "tatevik") else ctx_now  # a window, its kept positions, a page's slack
                 by = B * keys * kv_heads * 2 * dim * 2
                 kern["attention"]["algorithmic_bytes"] = by
                 kern["attention"]["frac_of_hbm_peak"] = round(by / (kern["attention"]["us_per_launch"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)
@@ -601,7 +642,7 @@ def main():
     ap.add_argument("--hybrid", choices=sorted(HYBRID_SIZES), default=None,
                     help="instead of the default workload: Lenisun / Senadra variants beside Llama at this size (prefill + decode)")
     ap.add_argument("--hybrid-models", default="llama,attn,mixed",
-                    help="comma list of llama, attn, mixed (Lenisun), senadra_attn, senadra, mananex_dense, mananex")
+                    help="comma list of llama, attn, mixed (Lenisun), senadra_attn, senadra, mananex_dense, mananex, tatevik_pair, tatevik")
     ap.add_argument("--prefill-batch", type=int, default=4)
     ap.add_argument("--prefill-len", type=int, default=1024)
     ap.add_argument("--prefill-reps", type=int, default=3)

@@ -327,6 +327,8 @@ def _write_and_attend(native, dev, dtype, q, k, v, talk, scale, window, rot, pie
     vp = torch.zeros((pages + 3, G, dv * 32), dtype=dtype, device=dev)
     order = torch.randperm(pages + 2, generator=torch.Generator().manual_seed(n))[:pages].to(torch.int32)
     bt = order.view(1, -1).to(dev)
+    from tgis_amd.utils.layers import workspace
+
     inv = torch.tensor([rot[0] ** (-2.0 * i / rot[1]) for i in range(rot[1] // 2)], dtype=torch.float32, device=dev) if rot[1] else None
     proj = torch.cat([q.reshape(n, -1), k.reshape(n, -1), v.reshape(n, -1)], 1).to(dtype).to(dev)
     outs, at = [], 0
@@ -337,7 +339,8 @@ def _write_and_attend(native, dev, dtype, q, k, v, talk, scale, window, rot, pie
         native.rope_rows_unit_kv_write(part, 0, H * dk, (H + G) * dk, inv, pos, slots, kp, vp, H, G, dk, dv, rot[1], eps)
         outs.append(native.attn_mixed_heads(part[:, :H * dk], kp, vp, bt, torch.tensor([at + c], dtype=torch.int32, device=dev),
                                             torch.tensor([0, c], dtype=torch.int32, device=dev), talk.to(dev), H, G, dk, dv, scale,
-                                            window=window, gate=None if gate is None else gate[at:at + c].to(dtype).to(dev), max_q_len=c))
+                                            window=window, gate=None if gate is None else gate[at:at + c].to(dtype).to(dev), max_q_len=c,
+                                            max_ctx=at + c, ws=workspace(dev)))  # single tokens take the key-split form
         at += c
     return torch.cat(outs)
 

@@ -75,10 +75,14 @@ __global__ __launch_bounds__(THREADS) void attn_mixed_heads_kernel(MixArgs a) {
     // running statistics of (head, query): read by the half wave that holds the head's keys, written by its first lane
     float* mrun = lsum + H * QT;                // [H][QT]
     float* lrun = mrun + H * QT;                // [H][QT]
+    float* mixs = lrun + H * QT;                // [H][H] the mixing matrix
     for (int e = tid; e < H * QT; e += THREADS) {
         mrun[e] = -INFINITY;
         lrun[e] = 0.f;
     }
+    for (int e = tid; e < H * H; e += THREADS) mixs[e] = a.mix[e];
+    // heads a thread mixes for its key: with many heads a column of raw scores is read once for HB of them
+    const int HB = H % 4 == 0 && H >= 32 ? 4 : (H % 2 == 0 && H >= 16 ? 2 : 1);
     float acc[OPT][QT];
 #pragma unroll
     for (int o = 0; o < OPT; ++o)
@@ -134,39 +138,51 @@ __global__ __launch_bounds__(THREADS) void attn_mixed_heads_kernel(MixArgs a) {
         }
         __syncthreads();
         // ---- mix over heads, mask, online softmax ----
-        for (int tr = 0; tr < trips; ++tr) {
-            const int pr = tid + tr * THREADS;
-            if (pr >= pairs) break;  // whole half waves leave together (pairs is a multiple of 32)
-            const int h = pr / PAGE, j = pr % PAGE;
-            float s[QT];
+        for (int pr = tid; pr < (H / HB) * PAGE; pr += THREADS) {  // whole half waves leave together
+            const int h0 = pr / PAGE * HB, j = pr % PAGE;
+            float s[4][QT];
 #pragma unroll
-            for (int qi = 0; qi < QT; ++qi) s[qi] = 0.f;
+            for (int hb = 0; hb < 4; ++hb)
+#pragma unroll
+                for (int qi = 0; qi < QT; ++qi) s[hb][qi] = 0.f;
             for (int g = 0; g < H; ++g) {
-                const float m = a.mix[h * H + g];
+                float r[QT];
 #pragma unroll
-                for (int qi = 0; qi < QT; ++qi) s[qi] = fmaf(m, raw[(g * QT + qi) * PAGE + j], s[qi]);
+                for (int qi = 0; qi < QT; ++qi) r[qi] = raw[(g * QT + qi) * PAGE + j];
+#pragma unroll
+                for (int hb = 0; hb < 4; ++hb)
+                    if (hb < HB) {
+                        const float m = mixs[(h0 + hb) * H + g];
+#pragma unroll
+                        for (int qi = 0; qi < QT; ++qi) s[hb][qi] = fmaf(m, r[qi], s[hb][qi]);
+                    }
             }
             const int key = key0 + j;
 #pragma unroll
-            for (int qi = 0; qi < QT; ++qi) {
-                const int pos = pos0 + qi;
-                const bool vis = qi < nq && key <= pos && (a.window <= 0 || pos - key < a.window);
-                float v = vis ? s[qi] : -INFINITY;
-                float mx = v;
+            for (int hb = 0; hb < 4; ++hb) {
+                if (hb >= HB) break;
+                const int h = h0 + hb;
 #pragma unroll
-                for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-                const float m_old = mrun[h * QT + qi];
-                const float m_new = fmaxf(m_old, mx);
-                const float p = vis ? expf(v - m_new) : 0.f;
-                float ps = p;
+                for (int qi = 0; qi < QT; ++qi) {
+                    const int pos = pos0 + qi;
+                    const bool vis = qi < nq && key <= pos && (a.window <= 0 || pos - key < a.window);
+                    float v = vis ? s[hb][qi] : -INFINITY;
+                    float mx = v;
 #pragma unroll
-                for (int o = 16; o > 0; o >>= 1) ps += __shfl_xor(ps, o, 64);
-                const float f = m_new == -INFINITY ? 1.f : expf(m_old - m_new);  // m_old = -inf: 0 (nothing summed yet)
-                pw[(h * QT + qi) * PAGE + j] = p;
-                if (j == 0) {
-                    fac[h * QT + qi] = f;
-                    lrun[h * QT + qi] = lrun[h * QT + qi] * f + ps;
-                    mrun[h * QT + qi] = m_new;
+                    for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+                    const float m_old = mrun[h * QT + qi];
+                    const float m_new = fmaxf(m_old, mx);
+                    const float p = vis ? expf(v - m_new) : 0.f;
+                    float ps = p;
+#pragma unroll
+                    for (int o = 16; o > 0; o >>= 1) ps += __shfl_xor(ps, o, 64);
+                    const float f = m_new == -INFINITY ? 1.f : expf(m_old - m_new);  // m_old = -inf: 0 (nothing summed yet)
+                    pw[(h * QT + qi) * PAGE + j] = p;
+                    if (j == 0) {
+                        fac[h * QT + qi] = f;
+                        lrun[h * QT + qi] = lrun[h * QT + qi] * f + ps;
+                        mrun[h * QT + qi] = m_new;
+                    }
                 }
             }
         }
@@ -220,9 +236,229 @@ __global__ __launch_bounds__(THREADS) void attn_mixed_heads_kernel(MixArgs a) {
     }
 }
 
+// ---- decode steps: one query token per sequence -------------------------------------------------------------------------------
+// A sequence's visible pages are dealt to `splits` workgroups (grid.x), so that a small batch still fills the chip; each leaves
+// unnormalised sums and softmax statistics of its pages in `part` ([split][token][H][dv + 2] fp32: sums, m, l) and
+// attn_mixed_combine_kernel merges them.  The R = H / G query heads that share a cached head are served together: a thread
+// that holds a key row (or a value channel's 32 tokens) uses it for all R of them, so a page is read once per workgroup.
+// MAXIT: (cached head, value channel) pairs a thread accumulates, R x MAXIT = 16.
+template <typename T, int R, int MAXIT>
+__global__ __launch_bounds__(THREADS) void attn_mixed_decode_kernel(MixArgs a, float* __restrict__ part, int splits, int64_t T_total) {
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    const int H = a.H, G = a.G, dk = a.dk, dv = a.dv;
+    const int b = blockIdx.y, sp = blockIdx.x, tid = threadIdx.x;
+    const int t = a.cu_q[b];
+    if (a.cu_q[b + 1] - t <= 0) return;
+    const int pos = a.ctx_lens[b] - 1;
+    const int lo = a.window > 0 ? max(pos - a.window + 1, 0) : 0;
+    const int p_lo = lo / PAGE, p_hi = pos / PAGE;
+    const int per = (p_hi - p_lo + splits) / splits;
+    const int pg0 = p_lo + sp * per, pg1 = min(pg0 + per - 1, p_hi);
+    const int dkp = (dk + 3) & ~3;
+    float* qs = smem;                 // [H][dkp]
+    float* raw = qs + H * dkp;        // [H][PAGE]
+    float* pw = raw + H * PAGE;       // [H][PAGE]
+    float* fac = pw + H * PAGE;       // [H]
+    float* mrun = fac + H;            // [H]
+    float* lrun = mrun + H;           // [H]
+    float* mixs = lrun + H;           // [H][H]
+    for (int e = tid; e < H * H; e += THREADS) mixs[e] = a.mix[e];
+    const T* q = reinterpret_cast<const T*>(a.q) + (int64_t)t * a.ldq;
+    for (int e = tid; e < H * dkp; e += THREADS) {
+        const int h = e / dkp, d = e - h * dkp;
+        qs[e] = d < dk ? (float)q[(int64_t)h * dk + d] * a.scale : 0.f;
+    }
+    for (int e = tid; e < H; e += THREADS) {
+        mrun[e] = -INFINITY;
+        lrun[e] = 0.f;
+    }
+    float acc[MAXIT][R];
+#pragma unroll
+    for (int i = 0; i < MAXIT; ++i)
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[i][r] = 0.f;
+    const T* kp = reinterpret_cast<const T*>(a.k_pool);
+    const T* vp = reinterpret_cast<const T*>(a.v_pool);
+    constexpr int VN = Vec16<T>::N;
+    typedef typename Vec16<T>::type VT;
+    const bool k_vec = dk % VN == 0;
+    const int items = G * dv;
+    __syncthreads();
+    for (int pg = pg0; pg <= pg1; ++pg) {
+        const int64_t page = a.bt[(int64_t)b * a.bt_ld + pg];
+        const int key0 = pg * PAGE;
+        // raw scores of the R heads of a cached head against one key row
+        for (int pr = tid; pr < G * PAGE; pr += THREADS) {
+            const int c = pr / PAGE, j = pr % PAGE;
+            const T* krow = kp + ((page * G + c) * PAGE + j) * (int64_t)dk;
+            float s[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) s[r] = 0.f;
+            if (key0 + j <= pos) {
+                if (k_vec) {
+                    for (int d = 0; d < dk; d += VN) {
+                        const VT kv = *reinterpret_cast<const VT*>(krow + d);
+#pragma unroll
+                        for (int r = 0; r < R; ++r) {
+                            const float* qq = qs + (c * R + r) * dkp + d;
+#pragma unroll
+                            for (int u = 0; u < VN; u += 4) {
+                                const f32x4 q4 = *reinterpret_cast<const f32x4*>(qq + u);
+                                s[r] = fmaf((float)kv[u], q4[0], s[r]);
+                                s[r] = fmaf((float)kv[u + 1], q4[1], s[r]);
+                                s[r] = fmaf((float)kv[u + 2], q4[2], s[r]);
+                                s[r] = fmaf((float)kv[u + 3], q4[3], s[r]);
+                            }
+                        }
+                    }
+                } else {
+                    for (int d = 0; d < dk; ++d) {
+                        const float kf = (float)krow[d];
+#pragma unroll
+                        for (int r = 0; r < R; ++r) s[r] = fmaf(kf, qs[(c * R + r) * dkp + d], s[r]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) raw[(c * R + r) * PAGE + j] = s[r];
+        }
+        __syncthreads();
+        for (int pr = tid; pr < H * PAGE; pr += THREADS) {
+            const int h = pr / PAGE, j = pr % PAGE;
+            float s = 0.f;
+            for (int g = 0; g < H; ++g) s = fmaf(mixs[h * H + g], raw[g * PAGE + j], s);
+            const int key = key0 + j;
+            const bool vis = key <= pos && key >= lo;
+            const float v = vis ? s : -INFINITY;
+            float mx = v;
+#pragma unroll
+            for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+            const float m_old = mrun[h];
+            const float m_new = fmaxf(m_old, mx);
+            const float p = vis ? expf(v - m_new) : 0.f;
+            float ps = p;
+#pragma unroll
+            for (int o = 16; o > 0; o >>= 1) ps += __shfl_xor(ps, o, 64);
+            pw[h * PAGE + j] = p;
+            if (j == 0) {
+                const float f = m_new == -INFINITY ? 1.f : expf(m_old - m_new);
+                fac[h] = f;
+                lrun[h] = lrun[h] * f + ps;
+                mrun[h] = m_new;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < MAXIT; ++i) {
+            const int it = tid + i * THREADS;
+            if (it < items) {
+                const int c = it / dv, col = it - c * dv;
+                const T* vrow = vp + ((page * G + c) * dv + col) * (int64_t)PAGE;
+                float vv[PAGE];
+#pragma unroll
+                for (int u = 0; u < PAGE; u += VN) {
+                    const VT v8 = *reinterpret_cast<const VT*>(vrow + u);
+#pragma unroll
+                    for (int w = 0; w < VN; ++w) vv[u + w] = (float)v8[w];
+                }
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const float* pp = pw + (c * R + r) * PAGE;
+                    float s = 0.f;
+#pragma unroll
+                    for (int u = 0; u < PAGE; u += 4) {
+                        const f32x4 p4 = *reinterpret_cast<const f32x4*>(pp + u);
+                        s += p4[0] * vv[u] + p4[1] * vv[u + 1] + p4[2] * vv[u + 2] + p4[3] * vv[u + 3];
+                    }
+                    acc[i][r] = acc[i][r] * fac[c * R + r] + s;
+                }
+            }
+        }
+        __syncthreads();
+    }
+    float* prow = part + ((int64_t)sp * T_total + t) * H * (dv + 2);
+#pragma unroll
+    for (int i = 0; i < MAXIT; ++i) {
+        const int it = tid + i * THREADS;
+        if (it < items) {
+            const int c = it / dv, col = it - c * dv;
+#pragma unroll
+            for (int r = 0; r < R; ++r) prow[(int64_t)(c * R + r) * (dv + 2) + col] = acc[i][r];
+        }
+    }
+    for (int h = tid; h < H; h += THREADS) {
+        prow[(int64_t)h * (dv + 2) + dv] = mrun[h];
+        prow[(int64_t)h * (dv + 2) + dv + 1] = lrun[h];
+    }
+}
+
+// out[t][h dv + c] = sum_s acc_s e^(m_s - m) / sum_s l_s e^(m_s - m), m = max_s m_s, times the gate.  grid (token, ceil(H / 4)): a
+// wave per head, its lanes over the splits for the statistics and over the value channels for the sums.
+template <typename T>
+__global__ __launch_bounds__(THREADS) void attn_mixed_combine_kernel(const float* __restrict__ part, int splits, int64_t T_total, MixArgs a) {
+    const int64_t t = blockIdx.x;
+    const int H = a.H, dv = a.dv;
+    const int h = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (h >= H) return;
+    const int64_t stride = T_total * H * (int64_t)(dv + 2);
+    const float* p0 = part + (t * H + h) * (int64_t)(dv + 2);
+    float m = -INFINITY;
+    for (int s = lane; s < splits; s += 64) m = fmaxf(m, p0[s * stride + dv]);
+    m = wave_max(m);
+    float den = 0.f;
+    for (int s = lane; s < splits; s += 64) {
+        const float ms = p0[s * stride + dv];
+        den += ms == -INFINITY ? 0.f : p0[s * stride + dv + 1] * expf(ms - m);
+    }
+    den = wave_sum(den);
+    T* out = reinterpret_cast<T*>(a.out);
+    const T* gate = reinterpret_cast<const T*>(a.gate);
+    for (int c = lane; c < dv; c += 64) {
+        float num = 0.f;
+        for (int s = 0; s < splits; ++s) {
+            const float ms = p0[s * stride + dv];
+            if (ms != -INFINITY) num = fmaf(p0[s * stride + c], expf(ms - m), num);
+        }
+        float v = num / den;
+        const int oc = h * dv + c;
+        if (gate) v *= 1.f / (1.f + expf(-(float)gate[t * a.ld_gate + oc]));
+        out[t * a.ld_out + oc] = (T)v;
+    }
+}
+
+template <typename T, int R>
+void launch_decode(const MixArgs& a, int64_t B, int64_t T_total, int splits, float* part, hipStream_t st) {
+    constexpr int MAXIT = 16 / R;
+    const int dkp = (a.dk + 3) & ~3;
+    const size_t lds = ((size_t)a.H * dkp + (size_t)2 * a.H * PAGE + (size_t)3 * a.H + (size_t)a.H * a.H) * sizeof(float);
+    if (lds > 48 * 1024)
+        (void)hipFuncSetAttribute((const void*)attn_mixed_decode_kernel<T, R, MAXIT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL((attn_mixed_decode_kernel<T, R, MAXIT>), dim3((unsigned)splits, (unsigned)B), dim3(THREADS), lds, st, a, part, splits, T_total);
+    hipLaunchKernelGGL(attn_mixed_combine_kernel<T>, dim3((unsigned)T_total, (unsigned)((a.H + 3) / 4)), dim3(THREADS), 0, st, part, splits, T_total, a);
+}
+
+template <typename T>
+bool try_decode(const MixArgs& a, int64_t B, int64_t T_total, int64_t max_ctx, void* ws, int64_t ws_bytes, hipStream_t st) {
+    const int R = a.H / a.G;
+    if (!ws || (R != 1 && R != 2 && R != 4 && R != 8 && R != 16)) return false;
+    const int64_t keys = a.window > 0 ? std::min<int64_t>(max_ctx, (int64_t)a.window + PAGE) : max_ctx;
+    const int pages = (int)cdiv64(std::max<int64_t>(keys, 1), PAGE) + (a.window > 0 ? 1 : 0);
+    int splits = (int)std::max<int64_t>(1, std::min<int64_t>(pages, 512 / std::max<int64_t>(B, 1)));
+    const int64_t per_split = T_total * a.H * (a.dv + 2) * (int64_t)sizeof(float);
+    splits = (int)std::min<int64_t>(splits, ws_bytes / std::max<int64_t>(per_split, 1));
+    if (splits < 1) return false;
+    float* part = reinterpret_cast<float*>(ws);
+    if (R == 1) launch_decode<T, 1>(a, B, T_total, splits, part, st);
+    else if (R == 2) launch_decode<T, 2>(a, B, T_total, splits, part, st);
+    else if (R == 4) launch_decode<T, 4>(a, B, T_total, splits, part, st);
+    else if (R == 8) launch_decode<T, 8>(a, B, T_total, splits, part, st);
+    else launch_decode<T, 16>(a, B, T_total, splits, part, st);
+    return true;
+}
+
 size_t lds_bytes(int QT, int H, int dk) {
     const int dkp = (dk + 3) & ~3;
-    return ((size_t)QT * H * dkp + (size_t)2 * H * QT * PAGE + (size_t)4 * H * QT) * sizeof(float);
+    return ((size_t)QT * H * dkp + (size_t)2 * H * QT * PAGE + (size_t)4 * H * QT + (size_t)H * H) * sizeof(float);
 }
 
 template <typename T, int QT, int OPT>
@@ -259,10 +495,11 @@ void launch(const MixArgs& a, int64_t B, int64_t max_q_len, hipStream_t st) {
 extern "C" int tgis_attn_mixed_heads(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
                                      int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B,
                                      const float* mix, const void* gate, int64_t ld_gate, void* out, int64_t ld_out,
-                                     int64_t max_q_len, int H, int G, int dk, int dv, float scale, int window, int dtype, void* stream) {
+                                     int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv, float scale,
+                                     int window, void* workspace, int64_t workspace_bytes, int dtype, void* stream) {
     TGIS_CHECK_ARG(q && k_pool && v_pool && block_tables && ctx_lens && cu_seqlens_q && mix && out, "tgis_attn_mixed_heads: null tensor");
     TGIS_CHECK_ARG(H >= 1 && G >= 1 && H % G == 0 && dk >= 1 && dv >= 1 && ldq >= (int64_t)H * dk && ld_out >= (int64_t)H * dv &&
-                       (!gate || ld_gate >= (int64_t)H * dv) && window >= 0 && max_q_len >= 1,
+                       (!gate || ld_gate >= (int64_t)H * dv) && window >= 0 && max_q_len >= 1 && max_ctx >= 1 && total_q >= 0,
                    "tgis_attn_mixed_heads: bad geometry (H %d, G %d, dk %d, dv %d)", H, G, dk, dv);
     TGIS_CHECK_ARG((int64_t)H * dv <= 16 * THREADS, "tgis_attn_mixed_heads: heads x value width up to %d (got %d x %d)", 16 * THREADS, H, dv);
     TGIS_CHECK_ARG(lds_bytes(1, H, dk) <= 150 * 1024, "tgis_attn_mixed_heads: heads x key width too large for one workgroup (%d x %d)", H, dk);
@@ -272,9 +509,18 @@ extern "C" int tgis_attn_mixed_heads(const void* q, int64_t ldq, const void* k_p
     TgisTimedScope timed(TGIS_OP_ATTN, st);
     const MixArgs a{q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, mix, gate, ld_gate, out, ld_out, H, G, dk, dv,
                     window, scale};
-    if (dtype == TGIS_F16) launch<f16>(a, B, max_q_len, st);
-    else if (dtype == TGIS_BF16) launch<bf16>(a, B, max_q_len, st);
-    else launch<float>(a, B, max_q_len, st);
+    // steps of single tokens (total_q <= B says so whatever max_q_len's bound is): the key-split form when the geometry allows
+    bool done = false;
+    if (max_q_len == 1 && total_q <= B) {
+        if (dtype == TGIS_F16) done = try_decode<f16>(a, B, total_q, max_ctx, workspace, workspace_bytes, st);
+        else if (dtype == TGIS_BF16) done = try_decode<bf16>(a, B, total_q, max_ctx, workspace, workspace_bytes, st);
+        else done = try_decode<float>(a, B, total_q, max_ctx, workspace, workspace_bytes, st);
+    }
+    if (!done) {
+        if (dtype == TGIS_F16) launch<f16>(a, B, max_q_len, st);
+        else if (dtype == TGIS_BF16) launch<bf16>(a, B, max_q_len, st);
+        else launch<float>(a, B, max_q_len, st);
+    }
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
 }

@@ -320,3 +320,95 @@ def mananex_tensors(config, seed: int, device="cpu", dtype=torch.bfloat16) -> Di
         t[f"l{i}.dwa"] = c.to(dtype)
     vec("final.norm", W)
     return t
+
+
+def tatevik_tensors(config, seed: int, device="cpu", dtype=torch.bfloat16, decay_rank: int = 64) -> Dict[str, torch.Tensor]:
+    """Seeded full Tatevik checkpoint in the family's tensor naming for a `TatevikConfig`: N(0, 1 / fan_in) projections, norm
+    gains around one, sublayer scales around 0.5, head-mixing matrices near the identity, step sizes and decays in the range a
+    trained model of the kind uses."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    W = config.width
+    t: Dict[str, torch.Tensor] = {}
+
+    def lin(name, n, k, gain=1.0):
+        t[name] = (torch.randn(n, k, generator=g, device=device) * gain * k ** -0.5).to(dtype)
+
+    def vec(name, n, mean=0.0, std=0.05):
+        t[name] = (mean + torch.randn(n, generator=g, device=device) * std).to(dtype)
+
+    taps = config.canon_taps
+    t["embed"] = torch.randn(config.vocab, W, generator=g, device=device).to(dtype)
+    if config.loop:
+        lin("loop.in", W, 2 * W)
+        vec("loop.step", int(config.loop["times"]) * W, 0.0, 0.1)
+        t["loop.step"] = t["loop.step"].view(-1, W)
+    for i, lay in enumerate(config.layers):
+        m, p = lay["mixer"], f"l{i}.mix"
+        vec(f"l{i}.norm1", W, 1.0)
+        vec(f"l{i}.ls1", W, 0.5, 0.1)
+        if taps:
+            t[f"l{i}.canon1"] = (torch.randn(W, taps, generator=g, device=device) * 0.3).to(dtype)
+        if lay["type"] == "mamba1":
+            inner, N, R, K = m["inner"], m["state"], m["dt_rank"], m["conv"]
+            lin(f"{p}.in", 2 * inner, W)
+            t[f"{p}.conv"] = (torch.randn(inner, K, generator=g, device=device) * 0.4).to(dtype)
+            vec(f"{p}.conv.b", inner, 0.0, 0.1)
+            lin(f"{p}.x", R + 2 * N, inner)
+            lin(f"{p}.dt", inner, R)
+            vec(f"{p}.dt.b", inner, -2.0, 1.0)
+            t[f"{p}.A_log"] = torch.log(torch.rand(inner, N, generator=g, device=device) * 8 + 0.5).to(dtype)
+            vec(f"{p}.D", inner, 1.0, 0.2)
+            lin(f"{p}.o", W, inner)
+        elif lay["type"] == "parallel":
+            a, q = m["left"], f"{p}.left"
+            H, dk = a["heads"], a["dim"]
+            G, dv = a.get("kv_heads", H), a.get("vdim", dk)
+            for n_, rows in (("q", H * dk), ("k", G * dk), ("v", G * dv)):
+                lin(f"{q}.{n_}", rows, W)
+                vec(f"{q}.{n_}.b", rows, 0.0, 0.1)
+            t[f"{q}.talk"] = (torch.eye(H, device=device) + torch.randn(H, H, generator=g, device=device) * (0.5 / H)).to(dtype)
+            lin(f"{q}.g", H * dv, W)
+            lin(f"{q}.o", W, H * dv)
+            vec(f"{q}.o.b", W, 0.0, 0.1)
+            r, q = m["right"], f"{p}.right"
+            Hr, dkr, dvr = r["heads"], r["dim"], r.get("vdim", r["dim"])
+            lin(f"{q}.q", Hr * dkr, W)
+            lin(f"{q}.k", Hr * dkr, W)
+            lin(f"{q}.v", Hr * dvr, W)
+            lin(f"{q}.g", Hr * dvr, W)
+            lin(f"{q}.o", W, Hr * dvr)
+            vec(f"{q}.norm", Hr * dvr, 1.0)
+            vec(f"{p}.left.out", W, 1.0)
+            vec(f"{p}.right.out", W, 1.0)
+        else:
+            H, dk, dv = m["heads"], m["dim"], m.get("vdim", m["dim"])
+            lin(f"{p}.q", H * dk, W)
+            lin(f"{p}.k", H * dk, W)
+            lin(f"{p}.v", H * dv, W)
+            lin(f"{p}.g", H * dv, W)
+            lin(f"{p}.o", W, H * dv)
+            vec(f"{p}.norm", dv, 1.0)
+            lin(f"{p}.a1", decay_rank, W)
+            lin(f"{p}.a2", H * dk, decay_rank)
+            vec(f"{p}.a2.b", H * dk, 3.0, 1.0)
+        f = lay.get("mlp")
+        if f:
+            q = f"l{i}.mlp"
+            vec(f"l{i}.ls2", W, 0.5, 0.1)
+            if taps:
+                t[f"l{i}.canon2"] = (torch.randn(W, taps, generator=g, device=device) * 0.3).to(dtype)
+            if f["kind"] == "dense":
+                lin(f"{q}.up", f["ff"], W)
+                lin(f"{q}.down", W, f["ff"])
+                t[f"{q}.act"] = torch.tensor([0.9, 0.3, -0.1, 0.05], device=device).to(dtype)
+            else:
+                E = f["router"]["experts"]
+                for e in range(E):
+                    lin(f"{q}.e{e}.gate", f["expert"]["ff"], W)
+                    lin(f"{q}.e{e}.up", f["expert"]["ff"], W)
+                    lin(f"{q}.e{e}.down", W, f["expert"]["ff"])
+                lin(f"{q}.router", E, W)
+                vec(f"{q}.correction", E, 0.0, 0.05)
+    vec("final.norm", W, 1.0)
+    lin("head", config.vocab, W)
+    return t

@@ -598,7 +598,7 @@ class MixedHeadAttention:
         gate = proj[:, cols[3]:cols[3] + self.H * self.dv] if self.has_gate else None
         return native.attn_mixed_heads(proj[:, cols[0]:cols[0] + self.H * self.dk], k_pool, v_pool, step.block_tables, step.ctx_lens,
                                        step.cu_seqlens_q, self.talk, self.H, self.G, self.dk, self.dv, self.scale, window=self.window,
-                                       gate=gate, max_q_len=step.max_q_len)
+                                       gate=gate, max_q_len=step.max_q_len, max_ctx=step.max_ctx, ws=workspace(proj.device))
 
 
 class DecayedLinearAttention:
