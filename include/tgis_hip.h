@@ -549,12 +549,13 @@ int tgis_rope_rows_unit_kv_write(void* proj, int64_t ld, int64_t q_col0, int64_t
  * s'_h = sum_g mix[h][g] s_g, mix [H][H] fp32; a query at position i sees keys j <= i with i - j < window (window 0: all);
  * out[t][h dv + c] is multiplied by sigmoid(gate[t][h dv + c]) when gate is given.  H dv <= 4096.  total_q: tokens of the step;
  * max_q_len, max_ctx: upper bounds (launch shaping only).  workspace (optional): scratch for the key-split form of steps of
- * single tokens (splits * total_q * H * (dv + 2) floats are used, as many splits as fit). */
+ * single tokens (splits * total_q * H * (dv + 2) floats are used, as many splits as fit).  impl 0: the launcher chooses
+ * (matrix-core form for prompt portions of two-byte models with dk % 16 == 0 and dv % 16 == 0); 1: the general kernel. */
 int tgis_attn_mixed_heads(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
                           int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B, const float* mix,
                           const void* gate, int64_t ld_gate, void* out, int64_t ld_out, int64_t total_q, int64_t max_q_len,
                           int64_t max_ctx, int H, int G, int dk, int dv, float scale, int window, void* workspace,
-                          int64_t workspace_bytes, int dtype, void* stream);
+                          int64_t workspace_bytes, int impl, int dtype, void* stream);
 /* Linear attention S <- diag(a) S + k v^T, o = S^T q per (sequence, head) on columns of proj [T, ld]:
  *   decay_mode 0: a = lower + (1 - lower) sigmoid(f + f_bias);  1: a = sigmoid(f + f_bias)^inv_tau;  2: a = head_decay[h];
  *   k at k_col0 (k_col0 < 0: k = 1 - a);  q_act / k_act / v_act != 0: SiLU on the projection;  q times q_scale;

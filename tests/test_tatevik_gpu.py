@@ -317,7 +317,7 @@ def test_selective_scan_and_its_state(gpu_device, dtype, inner, N):
 GEOMETRIES = [(6, 3, 32, 24), (8, 2, 48, 48), (4, 4, 16, 64), (2, 1, 128, 128), (3, 1, 10, 6), (32, 8, 64, 64)]
 
 
-def _write_and_attend(native, dev, dtype, q, k, v, talk, scale, window, rot, pieces, eps=1e-5, gate=None):
+def _write_and_attend(native, dev, dtype, q, k, v, talk, scale, window, rot, pieces, eps=1e-5, gate=None, impl=0):
     """q [n, H, dk], k [n, G, dk], v [n, G, dv] of one sequence go through rotation, unit norm and cache write, then
     attention, in the given portions; pages are dealt in a scrambled order.  Returns [n, H dv]."""
     n, H, dk = q.shape
@@ -340,7 +340,7 @@ def _write_and_attend(native, dev, dtype, q, k, v, talk, scale, window, rot, pie
         outs.append(native.attn_mixed_heads(part[:, :H * dk], kp, vp, bt, torch.tensor([at + c], dtype=torch.int32, device=dev),
                                             torch.tensor([0, c], dtype=torch.int32, device=dev), talk.to(dev), H, G, dk, dv, scale,
                                             window=window, gate=None if gate is None else gate[at:at + c].to(dtype).to(dev), max_q_len=c,
-                                            max_ctx=at + c, ws=workspace(dev)))  # single tokens take the key-split form
+                                            max_ctx=at + c, ws=workspace(dev), impl=impl))  # single tokens take the key-split form
         at += c
     return torch.cat(outs)
 
@@ -365,9 +365,10 @@ def test_mixed_head_attention_against_plain_softmax(gpu_device, dtype, geom, win
     qn = ref.rms_unit(ref.rotate_pairs(r16(q), pos, *rot), 1e-5)
     kn = ref.rms_unit(ref.rotate_pairs(r16(k), pos, *rot), 1e-5)
     want = ref.attend_mixed(qn, kn, r16(v), pos, talk.double(), 0.5, window).reshape(n, H * dv) * torch.sigmoid(r16(gate))
-    got = _write_and_attend(native, gpu_device, dtype, q, k, v, talk, 0.5, window, rot, [100, 2, 31, 33, 1, 1, 3, 40] + [1] * 19, gate=gate)
     tol = 2e-5 if dtype == torch.float32 else 0.03
-    assert float((got.double().cpu() - want).abs().max()) <= tol * float(want.abs().max())
+    for impl in (0, 1):  # the launcher's choice (matrix cores for portions of two-byte models), and the general kernel
+        got = _write_and_attend(native, gpu_device, dtype, q, k, v, talk, 0.5, window, rot, [100, 2, 31, 33, 1, 1, 3, 40] + [1] * 19, gate=gate, impl=impl)
+        assert float((got.double().cpu() - want).abs().max()) <= tol * float(want.abs().max()), impl
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

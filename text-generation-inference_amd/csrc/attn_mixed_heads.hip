@@ -14,6 +14,7 @@
 // cache dtype T is.  The same kernel serves prompt portions (QT up to 8) and decode steps (QT = 1).
 //
 // Cache pages: the "rows" layout of tgis_attn_varlen — k_pool[page][kv head][token][dk], v_pool[page][kv head][dv][token].
+#include <stdlib.h>
 #include <algorithm>
 #include "common.h"
 
@@ -283,44 +284,60 @@ __global__ __launch_bounds__(THREADS) void attn_mixed_decode_kernel(MixArgs a, f
     typedef typename Vec16<T>::type VT;
     const bool k_vec = dk % VN == 0;
     const int items = G * dv;
+    // heads per thread in the raw-score phase: R, or fewer (a power of two) while that gives more threads a key row
+    int RT = R;
+    while (RT > 1 && G * (R / RT) * PAGE * 2 <= THREADS) RT >>= 1;
     __syncthreads();
     for (int pg = pg0; pg <= pg1; ++pg) {
         const int64_t page = a.bt[(int64_t)b * a.bt_ld + pg];
         const int key0 = pg * PAGE;
-        // raw scores of the R heads of a cached head against one key row
-        for (int pr = tid; pr < G * PAGE; pr += THREADS) {
-            const int c = pr / PAGE, j = pr % PAGE;
+        // raw scores of a cached head's R query heads against one key row; with few cached heads the R heads are dealt to
+        // R / RT threads of RT heads each, so that the workgroup's threads all have a row
+        for (int pr = tid; pr < G * (R / RT) * PAGE; pr += THREADS) {
+            const int cs = pr / PAGE, j = pr % PAGE;
+            const int c = cs / (R / RT), h0 = c * R + (cs % (R / RT)) * RT;
             const T* krow = kp + ((page * G + c) * PAGE + j) * (int64_t)dk;
             float s[R];
 #pragma unroll
             for (int r = 0; r < R; ++r) s[r] = 0.f;
             if (key0 + j <= pos) {
                 if (k_vec) {
-                    for (int d = 0; d < dk; d += VN) {
-                        const VT kv = *reinterpret_cast<const VT*>(krow + d);
+                    // eight 16-byte pieces of the key row are asked for together (a piece at a time would cost a trip to memory each)
+                    for (int d0 = 0; d0 < dk; d0 += 8 * VN) {
+                        VT kv[8];
 #pragma unroll
-                        for (int r = 0; r < R; ++r) {
-                            const float* qq = qs + (c * R + r) * dkp + d;
+                        for (int e = 0; e < 8; ++e)
+                            if (d0 + e * VN < dk) kv[e] = *reinterpret_cast<const VT*>(krow + d0 + e * VN);
 #pragma unroll
-                            for (int u = 0; u < VN; u += 4) {
-                                const f32x4 q4 = *reinterpret_cast<const f32x4*>(qq + u);
-                                s[r] = fmaf((float)kv[u], q4[0], s[r]);
-                                s[r] = fmaf((float)kv[u + 1], q4[1], s[r]);
-                                s[r] = fmaf((float)kv[u + 2], q4[2], s[r]);
-                                s[r] = fmaf((float)kv[u + 3], q4[3], s[r]);
+                        for (int e = 0; e < 8; ++e)
+                            if (d0 + e * VN < dk) {
+#pragma unroll
+                                for (int r = 0; r < R; ++r)
+                                    if (r < RT) {
+                                        const float* qq = qs + (h0 + r) * dkp + d0 + e * VN;
+#pragma unroll
+                                        for (int u = 0; u < VN; u += 4) {
+                                            const f32x4 q4 = *reinterpret_cast<const f32x4*>(qq + u);
+                                            s[r] = fmaf((float)kv[e][u], q4[0], s[r]);
+                                            s[r] = fmaf((float)kv[e][u + 1], q4[1], s[r]);
+                                            s[r] = fmaf((float)kv[e][u + 2], q4[2], s[r]);
+                                            s[r] = fmaf((float)kv[e][u + 3], q4[3], s[r]);
+                                        }
+                                    }
                             }
-                        }
                     }
                 } else {
                     for (int d = 0; d < dk; ++d) {
                         const float kf = (float)krow[d];
 #pragma unroll
-                        for (int r = 0; r < R; ++r) s[r] = fmaf(kf, qs[(c * R + r) * dkp + d], s[r]);
+                        for (int r = 0; r < R; ++r)
+                            if (r < RT) s[r] = fmaf(kf, qs[(h0 + r) * dkp + d], s[r]);
                     }
                 }
             }
 #pragma unroll
-            for (int r = 0; r < R; ++r) raw[(c * R + r) * PAGE + j] = s[r];
+            for (int r = 0; r < R; ++r)
+                if (r < RT) raw[(h0 + r) * PAGE + j] = s[r];
         }
         __syncthreads();
         for (int pr = tid; pr < H * PAGE; pr += THREADS) {
@@ -443,7 +460,8 @@ bool try_decode(const MixArgs& a, int64_t B, int64_t T_total, int64_t max_ctx, v
     if (!ws || (R != 1 && R != 2 && R != 4 && R != 8 && R != 16)) return false;
     const int64_t keys = a.window > 0 ? std::min<int64_t>(max_ctx, (int64_t)a.window + PAGE) : max_ctx;
     const int pages = (int)cdiv64(std::max<int64_t>(keys, 1), PAGE) + (a.window > 0 ? 1 : 0);
-    int splits = (int)std::max<int64_t>(1, std::min<int64_t>(pages, 512 / std::max<int64_t>(B, 1)));
+    static const int64_t target_wgs = getenv("TGIS_MIXED_DECODE_WGS") ? atoll(getenv("TGIS_MIXED_DECODE_WGS")) : 512;
+    int splits = (int)std::max<int64_t>(1, std::min<int64_t>(pages, target_wgs / std::max<int64_t>(B, 1)));
     const int64_t per_split = T_total * a.H * (a.dv + 2) * (int64_t)sizeof(float);
     splits = (int)std::min<int64_t>(splits, ws_bytes / std::max<int64_t>(per_split, 1));
     if (splits < 1) return false;
@@ -454,6 +472,224 @@ bool try_decode(const MixArgs& a, int64_t B, int64_t T_total, int64_t max_ctx, v
     else if (R == 8) launch_decode<T, 8>(a, B, T_total, splits, part, st);
     else launch_decode<T, 16>(a, B, T_total, splits, part, st);
     return true;
+}
+
+// ---- prompt portions on the matrix cores (two-byte dtypes, dk % 16 == 0, dv % 16 == 0) ------------------------------------------
+// Workgroup = 16 consecutive query tokens of a sequence x all heads, NW waves; wave w owns heads w, w + NW, ...  Per page of 32
+// keys: raw scores S_g = Q_g K^T by 16x16x32 products (A = the query rows, B = the page's key rows, both 16-byte fragment loads
+// from memory; a lane of the accumulator holds key l % 16 of queries 4 (l / 16) .. + 3) into LDS in fp32; after a barrier every
+// wave mixes the H raw tiles into its own heads' tiles (a raw value read from LDS serves all of the wave's heads), masks, and
+// keeps the online softmax of its (head, query) rows in registers — a row's 32 keys live in 16 neighbouring lanes; the
+// weights go to LDS rounded to T as the A operand of O += P V, whose B operand is the channel-major value page (16 bytes = 8
+// tokens of a channel).  Scores, the mix, weights and statistics are fp32; only P is rounded for the last product.
+constexpr int RAW_ROW = 20;   // floats per KEY row of a raw tile (16 queries + 4: a lane's four queries are one 16-byte access)
+constexpr int P_ROW = 40;     // T elements per query row of a weight tile (80 bytes: 16-byte aligned, staggered)
+
+// the value of the lane N places further on in its row of 16 lanes (a data-parallel-primitive move: no trip through LDS); four of
+// them with N = 8, 4, 2, 1 leave a row's sum or maximum in all of its lanes
+template <int N> __device__ __forceinline__ float row_ror(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x120 + N, 0xF, 0xF, true));
+}
+
+template <typename T, int HW, int DVT>
+__global__ __launch_bounds__(512) void attn_mixed_mfma_kernel(MixArgs a) {
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    typedef typename Vec16<T>::type V8;
+    const int H = a.H, G = a.G, dk = a.dk, dv = a.dv, R = H / G;
+    const int NW = blockDim.x >> 6, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int lr = lane & 15, lg = lane >> 4;  // fragment row / column, and the group of 8 k-slots (or of 4 accumulator rows)
+    const int b = blockIdx.y;
+    const int t0 = a.cu_q[b], qlen = a.cu_q[b + 1] - t0;
+    const int first = blockIdx.x * 16;
+    if (first >= qlen) return;
+    const int nq = min(16, qlen - first);
+    const int pos0 = a.ctx_lens[b] - qlen + first;
+    float* raw = smem;                                          // [H][32 keys][RAW_ROW]
+    float* mixs = raw + H * 32 * RAW_ROW;                       // [H][H]
+    T* pb = reinterpret_cast<T*>(mixs + H * H);                 // [H][16][P_ROW]
+    for (int e = threadIdx.x; e < H * H; e += blockDim.x) mixs[e] = a.mix[e];
+    const int nvt = dv / 16;
+    f32x4 O[HW][DVT];
+    float mrun[HW][4], lrun[HW][4];
+#pragma unroll
+    for (int i = 0; i < HW; ++i) {
+#pragma unroll
+        for (int t = 0; t < DVT; ++t) O[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            mrun[i][u] = -INFINITY;
+            lrun[i][u] = 0.f;
+        }
+    }
+    const T* q = reinterpret_cast<const T*>(a.q) + (int64_t)(t0 + first + min(lr, nq - 1)) * a.ldq;  // rows past the tile repeat its last one
+    const T* kp = reinterpret_cast<const T*>(a.k_pool);
+    const T* vp = reinterpret_cast<const T*>(a.v_pool);
+    const int lo_first = a.window > 0 ? max(pos0 - a.window + 1, 0) : 0;
+    const int last_pos = pos0 + nq - 1;
+    __syncthreads();
+    for (int pg = lo_first / PAGE; pg <= last_pos / PAGE; ++pg) {
+        const int64_t page = a.bt[(int64_t)b * a.bt_ld + pg];
+        const int key0 = pg * PAGE;
+        // ---- raw scores of this wave's heads: per 32 key channels the fragments of all its heads are asked for together ----
+        f32x4 s0[HW], s1[HW];
+#pragma unroll
+        for (int i = 0; i < HW; ++i) s0[i] = s1[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int d0 = 0; d0 < dk; d0 += 32) {
+            const int d = d0 + lg * 8;
+            V8 qa[HW], k0[HW], k1[HW];
+#pragma unroll
+            for (int i = 0; i < HW; ++i) {
+                const int h = min(wave + NW * i, H - 1);
+                const T* krow = kp + ((page * G + h / R) * PAGE + lr) * (int64_t)dk;
+                qa[i] = k0[i] = k1[i] = V8{};
+                if (d < dk) {
+                    qa[i] = *reinterpret_cast<const V8*>(q + (int64_t)h * dk + d);
+                    k0[i] = *reinterpret_cast<const V8*>(krow + d);
+                    k1[i] = *reinterpret_cast<const V8*>(krow + (int64_t)16 * dk + d);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < HW; ++i) {
+                s0[i] = mfma16(qa[i], k0[i], s0[i]);
+                s1[i] = mfma16(qa[i], k1[i], s1[i]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < HW; ++i) {
+            const int h = wave + NW * i;
+            if (h < H) {
+                float* rt = raw + (h * 32 + lr) * RAW_ROW + lg * 4;  // key lr (and lr + 16), queries 4 lg .. + 3
+                *reinterpret_cast<f32x4*>(rt) = s0[i] * a.scale;
+                *reinterpret_cast<f32x4*>(rt + 16 * RAW_ROW) = s1[i] * a.scale;
+            }
+        }
+        __syncthreads();
+        // ---- mix, mask, online softmax of this wave's (head, query) rows ----
+        float sm[HW][8];
+#pragma unroll
+        for (int i = 0; i < HW; ++i)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) sm[i][u] = 0.f;
+        for (int g = 0; g < H; ++g) {
+            const float* rt = raw + (g * 32 + lr) * RAW_ROW + lg * 4;
+            const f32x4 ra = *reinterpret_cast<const f32x4*>(rt), rb = *reinterpret_cast<const f32x4*>(rt + 16 * RAW_ROW);
+            const float r[8] = {ra[0], ra[1], ra[2], ra[3], rb[0], rb[1], rb[2], rb[3]};
+#pragma unroll
+            for (int i = 0; i < HW; ++i) {
+                const int h = min(wave + NW * i, H - 1);
+                const float m = mixs[h * H + g];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) sm[i][u] = fmaf(m, r[u], sm[i][u]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < HW; ++i) {
+            const int h = wave + NW * i;
+            if (h < H) {
+                T* pt = pb + (h * 16 + lg * 4) * P_ROW + lr;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int qi = lg * 4 + u, pos = pos0 + qi;
+                    const int ka = key0 + lr, kb2 = ka + 16;
+                    const bool va = qi < nq && ka <= pos && (a.window <= 0 || pos - ka < a.window);
+                    const bool vb = qi < nq && kb2 <= pos && (a.window <= 0 || pos - kb2 < a.window);
+                    const float xa = va ? sm[i][u] : -INFINITY, xb = vb ? sm[i][4 + u] : -INFINITY;
+                    float mx = fmaxf(xa, xb);
+                    mx = fmaxf(mx, row_ror<8>(mx));
+                    mx = fmaxf(mx, row_ror<4>(mx));
+                    mx = fmaxf(mx, row_ror<2>(mx));
+                    mx = fmaxf(mx, row_ror<1>(mx));
+                    const float m_new = fmaxf(mrun[i][u], mx);
+                    const float pa = va ? expf(xa - m_new) : 0.f, pb2 = vb ? expf(xb - m_new) : 0.f;
+                    float ps = pa + pb2;
+                    ps += row_ror<8>(ps);
+                    ps += row_ror<4>(ps);
+                    ps += row_ror<2>(ps);
+                    ps += row_ror<1>(ps);
+                    const float f = m_new == -INFINITY ? 1.f : expf(mrun[i][u] - m_new);
+                    lrun[i][u] = lrun[i][u] * f + ps;
+                    mrun[i][u] = m_new;
+                    if (f != 1.f) {
+#pragma unroll
+                        for (int t = 0; t < DVT; ++t) O[i][t][u] *= f;
+                    }
+                    pt[u * P_ROW] = (T)pa;
+                    pt[u * P_ROW + 16] = (T)pb2;
+                }
+            }
+        }
+        __syncthreads();
+        // ---- weights x values ----
+#pragma unroll
+        for (int i = 0; i < HW; ++i) {
+            const int h = wave + NW * i;
+            if (h < H) {
+                const V8 pa = *reinterpret_cast<const V8*>(pb + (h * 16 + lr) * P_ROW + lg * 8);
+                const T* vrow = vp + ((page * G + h / R) * dv + lr) * (int64_t)PAGE + lg * 8;
+#pragma unroll
+                for (int t = 0; t < DVT; ++t)
+                    if (t < nvt) O[i][t] = mfma16(pa, *reinterpret_cast<const V8*>(vrow + (int64_t)t * 16 * PAGE), O[i][t]);
+            }
+        }
+    }
+    T* out = reinterpret_cast<T*>(a.out);
+    const T* gate = reinterpret_cast<const T*>(a.gate);
+#pragma unroll
+    for (int i = 0; i < HW; ++i) {
+        const int h = wave + NW * i;
+        if (h < H) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int qi = lg * 4 + u;
+                if (qi < nq) {
+                    const int64_t t = t0 + first + qi;
+                    const float inv = 1.f / lrun[i][u];
+#pragma unroll
+                    for (int tl = 0; tl < DVT; ++tl)
+                        if (tl < nvt) {
+                            const int oc = h * dv + tl * 16 + lr;
+                            float v = O[i][tl][u] * inv;
+                            if (gate) v *= 1.f / (1.f + expf(-(float)gate[t * a.ld_gate + oc]));
+                            out[t * a.ld_out + oc] = (T)v;
+                        }
+                }
+            }
+        }
+    }
+}
+
+template <typename T, int HW, int DVT>
+void launch_mfma_as(const MixArgs& a, int64_t B, int64_t max_q_len, int nw, hipStream_t st) {
+    const size_t lds = ((size_t)a.H * 32 * RAW_ROW + (size_t)a.H * a.H) * sizeof(float) + (size_t)a.H * 16 * P_ROW * sizeof(T);
+    if (lds > 48 * 1024)
+        (void)hipFuncSetAttribute((const void*)attn_mixed_mfma_kernel<T, HW, DVT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL((attn_mixed_mfma_kernel<T, HW, DVT>), dim3((unsigned)cdiv64(max_q_len, 16), (unsigned)B), dim3(64 * nw), lds, st, a);
+}
+
+template <typename T, int HW>
+bool launch_mfma_hw(const MixArgs& a, int64_t B, int64_t max_q_len, int nw, hipStream_t st) {
+    const int nvt = a.dv / 16;
+    if (nvt <= 2) launch_mfma_as<T, HW, 2>(a, B, max_q_len, nw, st);
+    else if (nvt <= 4) launch_mfma_as<T, HW, 4>(a, B, max_q_len, nw, st);
+    else if (nvt <= 8) launch_mfma_as<T, HW, 8>(a, B, max_q_len, nw, st);
+    else if (nvt <= 16 && HW <= 2) launch_mfma_as<T, HW, (HW <= 2 ? 16 : 2)>(a, B, max_q_len, nw, st);
+    else return false;
+    return true;
+}
+
+// up to 8 heads: four waves of up to two heads; up to 32: eight waves of up to four (a wave's accumulators stay within 32
+// tiles of 16 x 16); false if the geometry is not served
+template <typename T>
+bool try_mfma(const MixArgs& a, int64_t B, int64_t max_q_len, hipStream_t st) {
+    if (a.dk % 16 || a.dv % 16 || a.dv > 256 || a.ldq % 8 || a.H > 32) return false;
+    if ((((uintptr_t)a.q) & 15) || (((uintptr_t)a.k_pool) & 15) || (((uintptr_t)a.v_pool) & 15)) return false;
+    const size_t lds = ((size_t)a.H * 32 * RAW_ROW + (size_t)a.H * a.H) * sizeof(float) + (size_t)a.H * 16 * P_ROW * sizeof(T);
+    if (lds > 150 * 1024) return false;
+    const int nw = a.H > 8 ? 8 : 4;
+    const int hw = (a.H + nw - 1) / nw;
+    if (hw <= 1) return launch_mfma_hw<T, 1>(a, B, max_q_len, nw, st);
+    if (hw <= 2) return launch_mfma_hw<T, 2>(a, B, max_q_len, nw, st);
+    return launch_mfma_hw<T, 4>(a, B, max_q_len, nw, st);
 }
 
 size_t lds_bytes(int QT, int H, int dk) {
@@ -496,7 +732,7 @@ extern "C" int tgis_attn_mixed_heads(const void* q, int64_t ldq, const void* k_p
                                      int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B,
                                      const float* mix, const void* gate, int64_t ld_gate, void* out, int64_t ld_out,
                                      int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv, float scale,
-                                     int window, void* workspace, int64_t workspace_bytes, int dtype, void* stream) {
+                                     int window, void* workspace, int64_t workspace_bytes, int impl, int dtype, void* stream) {
     TGIS_CHECK_ARG(q && k_pool && v_pool && block_tables && ctx_lens && cu_seqlens_q && mix && out, "tgis_attn_mixed_heads: null tensor");
     TGIS_CHECK_ARG(H >= 1 && G >= 1 && H % G == 0 && dk >= 1 && dv >= 1 && ldq >= (int64_t)H * dk && ld_out >= (int64_t)H * dv &&
                        (!gate || ld_gate >= (int64_t)H * dv) && window >= 0 && max_q_len >= 1 && max_ctx >= 1 && total_q >= 0,
@@ -515,6 +751,11 @@ extern "C" int tgis_attn_mixed_heads(const void* q, int64_t ldq, const void* k_p
         if (dtype == TGIS_F16) done = try_decode<f16>(a, B, total_q, max_ctx, workspace, workspace_bytes, st);
         else if (dtype == TGIS_BF16) done = try_decode<bf16>(a, B, total_q, max_ctx, workspace, workspace_bytes, st);
         else done = try_decode<float>(a, B, total_q, max_ctx, workspace, workspace_bytes, st);
+    }
+    // prompt portions of two-byte models: the matrix-core form (impl 1 keeps the general kernel for comparisons)
+    if (!done && max_q_len > 2 && impl != 1) {
+        if (dtype == TGIS_F16) done = try_mfma<f16>(a, B, max_q_len, st);
+        else if (dtype == TGIS_BF16) done = try_mfma<bf16>(a, B, max_q_len, st);
     }
     if (!done) {
         if (dtype == TGIS_F16) launch<f16>(a, B, max_q_len, st);

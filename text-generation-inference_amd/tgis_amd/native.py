@@ -146,7 +146,7 @@ SIGNATURES = {
     "tgis_rope_rows_unit_kv_write": (_c_int, [_vp, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp, _c_i64, _c_int, _c_int, _c_int,
                                               _c_int, _c_int, _c_f, _c_int, _vp]),
     "tgis_attn_mixed_heads": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64,
-                                       _c_i64, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _vp, _c_i64, _c_int, _vp]),
+                                       _c_i64, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _vp, _c_i64, _c_int, _c_int, _vp]),
     "tgis_linear_scan": (_c_int, [_vp, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _c_int, _c_f, _c_int, _c_int, _c_int, _c_f,
                                   _vp, _c_int, _vp, _c_i64, _c_int, _vp, _vp, _vp, _vp, _vp, _c_i64, _c_f, _c_i64, _c_i64, _c_i64,
                                   _c_int, _c_int, _c_int, _c_f, _vp, _c_int, _vp]),
@@ -1334,7 +1334,8 @@ def rope_rows_unit_kv_write(proj, q_col0: int, k_col0: int, v_col0: int, inv_fre
 
 
 def attn_mixed_heads(q, k_pool, v_pool, block_tables, ctx_lens, cu_seqlens_q, mix, H: int, G: int, dk: int, dv: int, scale: float,
-                     window: int = 0, gate=None, out=None, max_q_len: int = 1, max_ctx: int = 1, ws: Optional[Workspace] = None):
+                     window: int = 0, gate=None, out=None, max_q_len: int = 1, max_ctx: int = 1, ws: Optional[Workspace] = None,
+                     impl: int = 0):
     """Softmax attention over the paged cache with the heads' scores mixed by mix [H, H] (fp32) before the softmax; q [T, H dk]
     (a view with unit column stride), gate [T, H dv] or None -> [T, H dv].  ws: scratch for the key-split form of decode steps."""
     assert q.dim() == 2 and q.stride(1) == 1 and block_tables.dim() == 2 and mix.shape == (H, H) and mix.is_contiguous()
@@ -1348,7 +1349,7 @@ def attn_mixed_heads(q, k_pool, v_pool, block_tables, ctx_lens, cu_seqlens_q, mi
         _i32(ctx_lens, "ctx_lens"), _i32(cu_seqlens_q, "cu_seqlens_q"), ctx_lens.shape[0], _f32(mix, "mix"), _ptr(gate),
         gate.stride(0) if gate is not None else 0, _ptr(out), out.stride(0), T, max(int(max_q_len), 1), max(int(max_ctx), 1), H, G, dk, dv,
         float(scale), int(window), (ws.ptr + 4096) if ws is not None else None, (ws.nbytes - 4096) if ws is not None else 0,
-        dtype_code3(q.dtype), _stream()), "tgis_attn_mixed_heads")
+        int(impl), dtype_code3(q.dtype), _stream()), "tgis_attn_mixed_heads")
     return out
 
 
