@@ -8,7 +8,7 @@
 // projection before its bias.  The state [inner][N] of a sequence lives in a slot (fp32), is read when the step does not start
 // at position 0 and written back.
 //
-// Workgroup = (sequence, CW = 256 / L channels): L neighbouring lanes share a channel, lane l of them keeps states
+// Workgroup = (sequence, CW = threads / L channels; 64 .. 256 threads, fewer when the step has few sequences): L neighbouring lanes share a channel, lane l of them keeps states
 // l SPT .. l SPT + SPT - 1 in registers (L a power of two, SPT = ceil(N / L) <= 8).  Tokens go through LDS in stages of TS: the
 // stage's B | C rows and the channels' step sizes and inputs (softplus applied once per (token, channel), not per state), then a
 // sequential walk over the stage with the read-out summed over the channel's lanes by shuffles; the stage's outputs leave
@@ -43,11 +43,18 @@ struct SelArgs {
 };
 
 __device__ __forceinline__ float softplus_f32(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+// e^(d a) per state and token is what the walk spends its time on: where the model is served in two bytes it is the hardware's
+// base-two exponential (a few units in the last place of fp32) on a transition that was scaled by log2(e) once; fp32 serving
+// takes the library's.
+template <typename T> __device__ __forceinline__ float decay_of(float d, float a) {
+    if (sizeof(T) == 4) return expf(d * a);
+    return __builtin_amdgcn_exp2f(d * a);
+}
 
 template <typename T>
 __global__ __launch_bounds__(256) void selective_scan_kernel(SelArgs a) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
-    const int N = a.N, L = a.L, CW = 256 / L;
+    const int N = a.N, L = a.L, NT = blockDim.x, CW = NT / L;
     const int Np = L * SPT;
     float* Bs = smem;                 // [TS][Np]
     float* Cs = Bs + TS * Np;         // [TS][Np]
@@ -68,7 +75,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(SelArgs a) {
         const int n = l * SPT + r;
         const bool ok = live && n < N;
         s[r] = (ok && !fresh) ? S[n] : 0.f;
-        A[r] = ok ? -expf(a.A_log[(int64_t)c * N + n]) : 0.f;
+        A[r] = ok ? -expf(a.A_log[(int64_t)c * N + n]) * (sizeof(T) == 4 ? 1.f : 1.4426950408889634f) : 0.f;
     }
     const float Dc = live ? a.D[c] : 0.f;
     const T* x = reinterpret_cast<const T*>(a.x);
@@ -77,13 +84,13 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(SelArgs a) {
     T* out = reinterpret_cast<T*>(a.out);
     for (int base = 0; base < qlen; base += TS) {
         const int n_t = min(TS, qlen - base);
-        for (int e = tid; e < n_t * Np; e += 256) {
+        for (int e = tid; e < n_t * Np; e += NT) {
             const int tt = e / Np, n = e - tt * Np;
             const T* row = bc + (int64_t)(t0 + base + tt) * a.ld_bc;
             Bs[e] = n < N ? (float)row[a.b_col0 + n] : 0.f;
             Cs[e] = n < N ? (float)row[a.c_col0 + n] : 0.f;
         }
-        for (int e = tid; e < n_t * CW; e += 256) {
+        for (int e = tid; e < n_t * CW; e += NT) {
             const int tt = e / CW, cc = blockIdx.y * CW + e - tt * CW;
             float d = 0.f, xv = 0.f;
             if (cc < a.inner) {
@@ -108,7 +115,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(SelArgs a) {
                 const f32x4 c4 = *reinterpret_cast<const f32x4*>(Cr + r4);
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    s[r4 + u] = fmaf(expf(d * A[r4 + u]), s[r4 + u], dx * b4[u]);
+                    s[r4 + u] = fmaf(decay_of<T>(d, A[r4 + u]), s[r4 + u], dx * b4[u]);
                     y = fmaf(s[r4 + u], c4[u], y);
                 }
             }
@@ -116,7 +123,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(SelArgs a) {
             if (l == 0) ys[tt * CW + ch] = fmaf(Dc, xv, y);
         }
         __syncthreads();
-        for (int e = tid; e < n_t * CW; e += 256) {
+        for (int e = tid; e < n_t * CW; e += NT) {
             const int tt = e / CW, cc = blockIdx.y * CW + e - tt * CW;
             if (cc < a.inner) {
                 const int64_t t = t0 + base + tt;
@@ -152,14 +159,17 @@ extern "C" int tgis_selective_scan(const void* x, int64_t ld_x, const void* dt, 
     TgisTimedScope timed(TGIS_OP_SCAN, st);
     int L = 1;
     while (L * SPT < N) L <<= 1;
-    const int CW = 256 / L;
+    // few (sequence, channel block) pairs: smaller workgroups, so that the chip's compute units all get one
+    int threads = 256;
+    while (threads > 64 && threads / 2 >= L && B * cdiv64(inner, threads / L) < 512) threads >>= 1;
+    const int CW = threads / L;
     const SelArgs a{x, ld_x, dt, ld_dt, dt_f32, dt_bias, bc, ld_bc, b_col0, c_col0, z, ld_z, A_log, D, state, state_slots, cu_seqlens_q,
                     positions, out, ld_out, (int)inner, N, L};
     const size_t lds = ((size_t)2 * TS * L * SPT + (size_t)3 * TS * CW) * sizeof(float);
     const dim3 grid((unsigned)B, (unsigned)cdiv64(inner, CW));
-    if (dtype == TGIS_F16) hipLaunchKernelGGL(selective_scan_kernel<f16>, grid, dim3(256), lds, st, a);
-    else if (dtype == TGIS_BF16) hipLaunchKernelGGL(selective_scan_kernel<bf16>, grid, dim3(256), lds, st, a);
-    else hipLaunchKernelGGL(selective_scan_kernel<float>, grid, dim3(256), lds, st, a);
+    if (dtype == TGIS_F16) hipLaunchKernelGGL(selective_scan_kernel<f16>, grid, dim3(threads), lds, st, a);
+    else if (dtype == TGIS_BF16) hipLaunchKernelGGL(selective_scan_kernel<bf16>, grid, dim3(threads), lds, st, a);
+    else hipLaunchKernelGGL(selective_scan_kernel<float>, grid, dim3(threads), lds, st, a);
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
 }
