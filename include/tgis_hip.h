@@ -581,12 +581,13 @@ int tgis_causal_conv(const void* x, int64_t ld_x, int x_f32, const float* w, con
  *   d = softplus(dt[t][c] + dt_bias[c]);  S[c][n] <- exp(-d exp(A_log[c][n])) S[c][n] + d x[t][c] B[t][n];
  *   out[t][c] = (sum_n S[c][n] C[t][n] + D[c] x[t][c]) silu(z[t][c]).
  * x, z, out [T, >= inner] and bc [T, ld_bc] (B at b_col0, C at c_col0, N columns each) of `dtype`; dt fp32 (dt_f32) or `dtype`;
- * state [slots][inner][N] fp32, read unless the step starts at position 0, written back.  N <= 128. */
+ * state [slots][inner][N] fp32, read unless the step starts at position 0, written back.  N <= 128.  max_q_len: an upper bound
+ * of a sequence's run in the step (launch shaping only). */
 int tgis_selective_scan(const void* x, int64_t ld_x, const void* dt, int64_t ld_dt, int dt_f32, const float* dt_bias,
                         const void* bc, int64_t ld_bc, int64_t b_col0, int64_t c_col0, const void* z, int64_t ld_z,
                         const float* A_log, const float* D, float* state, const int32_t* state_slots,
                         const int32_t* cu_seqlens_q, const int32_t* positions, void* out, int64_t ld_out, int64_t B,
-                        int64_t inner, int N, int dtype, void* stream);
+                        int64_t max_q_len, int64_t inner, int N, int dtype, void* stream);
 /* x_out = x_in + s1 * a + s2 * b + v  (each term optional; s1, s2, v [W] fp32; a, b [rows, ld] fp32 or `dtype`), and
  * h = norm(x_out) * w with norm the mean-free layer norm (mean_free) or the RMS norm, eps inside the root; h fp32 (h_f32) or
  * `dtype`; w NULL: no norm.  x_out may alias x_in. */

@@ -153,7 +153,7 @@ SIGNATURES = {
     "tgis_causal_conv": (_c_int, [_vp, _c_i64, _c_int, _vp, _vp, _c_int, _vp, _c_i64, _vp, _vp, _vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64,
                                   _c_i64, _c_int, _c_int, _c_int, _c_int, _vp]),
     "tgis_selective_scan": (_c_int, [_vp, _c_i64, _vp, _c_i64, _c_int, _vp, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _vp, _vp, _vp, _vp,
-                                     _vp, _vp, _vp, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _vp]),
+                                     _vp, _vp, _vp, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _vp]),
     "tgis_scaled_residual_norm": (_c_int, [_vp, _vp, _vp, _c_i64, _c_int, _vp, _vp, _c_i64, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_i64,
                                            _c_i64, _c_f, _c_int, _c_int, _vp]),
     "tgis_rms_pair_mean": (_c_int, [_vp, _c_i64, _c_int, _vp, _c_f, _vp, _c_i64, _c_int, _vp, _c_f, _vp, _c_i64, _c_i64, _c_f, _c_int, _vp]),
@@ -1395,7 +1395,8 @@ def causal_conv(x, w, bias, tail, state_slots, cu_seqlens_q, positions, out_dtyp
     return out
 
 
-def selective_scan(x, dt, dt_bias, bc, b_col0: int, c_col0: int, z, A_log, D, state, state_slots, cu_seqlens_q, positions, N: int):
+def selective_scan(x, dt, dt_bias, bc, b_col0: int, c_col0: int, z, A_log, D, state, state_slots, cu_seqlens_q, positions, N: int,
+                   max_q_len: int = 0):
     """x, z [T, inner] views, dt [T, inner] (fp32 or the activation dtype), bc [T, ld] with B | C at their columns -> [T, inner]."""
     T, inner = x.shape
     assert all(t.stride(1) == 1 for t in (x, dt, bc, z)) and z.shape == x.shape and dt.shape == x.shape
@@ -1405,7 +1406,8 @@ def selective_scan(x, dt, dt_bias, bc, b_col0: int, c_col0: int, z, A_log, D, st
         _ptr(x), x.stride(0), _ptr(dt), dt.stride(0), int(dt.dtype == torch.float32 and x.dtype != torch.float32), _f32(dt_bias, "dt_bias"),
         _ptr(bc), bc.stride(0), b_col0, c_col0, _ptr(z), z.stride(0), _f32(A_log, "A_log"), _f32(D, "D"), _ptr(state),
         _i32(state_slots, "state_slots"), _i32(cu_seqlens_q, "cu_seqlens_q"), _i32(positions, "positions"), _ptr(out), out.stride(0),
-        state_slots.shape[0], inner, N, dtype_code3(x.dtype), _stream()), "tgis_selective_scan")
+        state_slots.shape[0], int(max_q_len) if max_q_len > 0 else max(T, 1), inner, N, dtype_code3(x.dtype), _stream()),
+        "tgis_selective_scan")
     return out
 
 

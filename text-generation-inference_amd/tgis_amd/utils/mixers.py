@@ -564,7 +564,7 @@ class SelectiveScanMixer:
         low = self.x_proj(x)
         dt = self.dt_proj(_view_for_gemm(low[:, self.dt_col:self.dt_col + self.R]), out_f32=True)
         y = native.selective_scan(x, dt, self.dt_bias, low, self.b_col, self.c_col, xz[:, self.inner:], self.A_log, self.D, state,
-                                  step.state_slots, step.cu_seqlens_q, position_ids, self.N)
+                                  step.state_slots, step.cu_seqlens_q, position_ids, self.N, max_q_len=step.max_q_len)
         return self.o(y, out_f32=True)
 
 
