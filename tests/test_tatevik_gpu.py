@@ -182,9 +182,9 @@ OTHER_SHAPES = {
                                          tiny.pair_layer(left=tiny.attention_part(heads=2, kv_heads=1, dim=12, vdim=20, window=1, rot_dims=4),
                                                          right=tiny.fixed_decay_part(heads=1, dim=8, vdim=8, decay=(0.9,)))],
                                  width=24, vocab=33, taps=2, loop={"start": 0, "stop": 2, "times": 2}),
-    "one_pass_one_tap": dict(layers=[tiny.scan_layer(inner=40, state=24, dt_rank=16, conv=3, mlp=tiny.moe_mlp(experts=9, top=4, ff=24, groups=3, keep=2)),
-                                     tiny.channel_decay_layer(heads=5, dim=12, vdim=20, tau=16.0, rank=4, mlp=tiny.dense_mlp(30)),
-                                     tiny.pair_layer(left=tiny.attention_part(heads=8, kv_heads=2, dim=24, vdim=8, window=33, rot_dims=0),
+    "one_pass_one_tap": dict(layers=[tiny.scan_layer(inner=40, state=20, dt_rank=12, conv=3, mlp=tiny.moe_mlp(experts=9, top=4, ff=24, groups=3, keep=2)),
+                                     tiny.channel_decay_layer(heads=5, dim=12, vdim=20, tau=12.0, rank=4, mlp=tiny.dense_mlp(30)),
+                                     tiny.pair_layer(left=tiny.attention_part(heads=8, kv_heads=4, dim=24, vdim=8, window=33, rot_dims=0),
                                                      right=tiny.fixed_decay_part(heads=4, dim=16, vdim=12, decay=(0.3, 0.8, 0.97, 1.0)))],
                              width=56, vocab=64, taps=1, loop={"start": 1, "stop": 3, "times": 1}),
     "odd_widths": dict(layers=[tiny.pair_layer(left=tiny.attention_part(heads=3, kv_heads=3, dim=10, vdim=6, window=64, rot_dims=6),
@@ -194,7 +194,7 @@ OTHER_SHAPES = {
                        width=36, vocab=41, taps=5, loop={"start": 2, "stop": 3, "times": 4}),
     "wide_heads": dict(layers=[tiny.pair_layer(left=tiny.attention_part(heads=4, kv_heads=2, dim=128, vdim=64, scale=0.08, window=70, rot_dims=64),
                                                right=tiny.fixed_decay_part(heads=2, dim=128, vdim=64, decay=(0.9, 0.99)), mlp=tiny.dense_mlp(128)),
-                               tiny.channel_decay_layer(heads=2, dim=64, vdim=128, tau=16.0, rank=16),
+                               tiny.channel_decay_layer(heads=2, dim=64, vdim=128, tau=10.0, rank=16),
                                tiny.scan_layer(inner=256, state=64, dt_rank=8, conv=4)],
                        width=128, vocab=80, taps=3, loop={"start": 0, "stop": 1, "times": 2}),
 }
@@ -284,7 +284,7 @@ def test_causal_convolution_through_its_tail(gpu_device, dtype, taps, sets, act)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("inner,N", [(96, 12), (40, 1), (300, 16), (64, 24), (33, 128), (70, 9)])
+@pytest.mark.parametrize("inner,N", [(96, 12), (40, 1), (300, 16), (64, 20), (33, 128), (70, 9)])
 def test_selective_scan_and_its_state(gpu_device, dtype, inner, N):
     from tgis_amd import native
 
@@ -314,7 +314,7 @@ def test_selective_scan_and_its_state(gpu_device, dtype, inner, N):
     assert float((state[1].double().cpu() - S).abs().max()) <= 2e-5 * float(S.abs().max()) and float(state[0].min()) == 55.0
 
 
-GEOMETRIES = [(6, 3, 32, 24), (8, 2, 48, 48), (4, 4, 16, 64), (2, 1, 128, 128), (3, 1, 10, 6), (32, 8, 64, 64)]
+GEOMETRIES = [(6, 3, 32, 24), (8, 2, 80, 48), (4, 4, 16, 64), (2, 1, 128, 128), (3, 1, 10, 6), (32, 8, 64, 64)]
 
 
 def _write_and_attend(native, dev, dtype, q, k, v, talk, scale, window, rot, pieces, eps=1e-5, gate=None, impl=0):
@@ -347,7 +347,7 @@ def _write_and_attend(native, dev, dtype, q, k, v, talk, scale, window, rot, pie
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("geom", GEOMETRIES)
-@pytest.mark.parametrize("window", [0, 1, 33, 72, 200])
+@pytest.mark.parametrize("window", [0, 1, 33, 70, 200])
 def test_mixed_head_attention_against_plain_softmax(gpu_device, dtype, geom, window):
     """Rotation, unit norm, cache write and attention with mixed heads, a window and a gate, in prompt portions and single
     tokens over scrambled pages, against the plain form."""
@@ -372,7 +372,7 @@ def test_mixed_head_attention_against_plain_softmax(gpu_device, dtype, geom, win
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("geom", [(6, 3, 32, 24), (8, 2, 48, 48)])
+@pytest.mark.parametrize("geom", [(6, 3, 32, 24), (8, 2, 80, 48)])
 @pytest.mark.parametrize("window", [40, 64, 97])
 def test_attention_finds_a_planted_key_inside_its_window_only(gpu_device, dtype, geom, window):
     """One key among 700 points where every query points, and its value is far from all others: a query sees it iff it lies in
@@ -417,7 +417,7 @@ def test_linear_attention_scan_and_its_state(gpu_device, dtype, heads, dim, vdim
     v, gt = P[:, cols[2]:cols[2] + H * dv].view(n, H, dv), P[:, cols[3]:cols[3] + H * dv]
     S0 = torch.zeros(H, dk, dv, dtype=D)
     if form == "head":
-        decay = torch.linspace(0.6, 0.999, H)
+        decay = torch.linspace(0.6, 0.995, H)
         gain = 1 + 0.2 * torch.randn(H * dv, generator=g)
         o, S = ref.linear_attention(ref.silu(q), ref.silu(k), ref.silu(v), decay.double().view(1, H, 1).expand(n, H, dk), S0)
         want = ref.rms_unit(o.reshape(n, H * dv), 1e-5) * gain.double() * torch.sigmoid(gt)
@@ -448,7 +448,7 @@ def test_linear_attention_scan_and_its_state(gpu_device, dtype, heads, dim, vdim
 
 
 def test_linear_attention_keeps_a_far_write(gpu_device):
-    """A key written at the first position and read 600 tokens later through a decay of 0.999 per step, among small writes."""
+    """A key written at the first position and read 600 tokens later through a decay of 0.998 per step, among small writes."""
     from tgis_amd import native
 
     dev, n, dk, dv = gpu_device, 601, 16, 16
@@ -459,9 +459,9 @@ def test_linear_attention_keeps_a_far_write(gpu_device):
     state = torch.zeros(1, 1, dk, dv, device=dev)
     st = _Step([0], [n], [0], dev)
     scratch_free = native.linear_scan(proj, 0, dk, -1, 2 * dk, state, st.slots, st.cu, st.pos, 1, dk, dv, 1e-12, torch.ones(dv, device=dev) * dv ** -0.5,
-                                      decay_mode=2, head_decay=torch.tensor([0.999], device=dev), q_act=True, k_act=True, v_act=True,
+                                      decay_mode=2, head_decay=torch.tensor([0.998], device=dev), q_act=True, k_act=True, v_act=True,
                                       norm_rows=True, gate=proj[:, 2 * dk + dv:], gate_act=1, max_q_len=n)
-    assert abs(float(state[0, 0, 3, 5]) / (10.0 * 10.0 * 0.999 ** 600) - 1) < 1e-3
+    assert abs(float(state[0, 0, 3, 5]) / (10.0 * 10.0 * 0.998 ** 600) - 1) < 1e-3
     assert abs(float(scratch_free[n - 1, 5]) - 0.5) < 1e-3  # the row's only entry, normed to one, times sigmoid(0)
 
 
@@ -583,7 +583,7 @@ def test_trace_runner_replays_a_schedule(gpu_device, tmp_path, dtype):
     from safetensors.torch import save_file
 
     layers = [tiny.pair_layer(left=tiny.attention_part(heads=8, kv_heads=4, dim=16, vdim=32, scale=0.25, window=20, rot_dims=4),
-                              right=tiny.fixed_decay_part(heads=4, dim=8, vdim=16, decay=(0.5, 0.8, 0.95, 0.999)), mlp=tiny.moe_mlp(experts=4, top=2, ff=32, groups=2, keep=1)),
+                              right=tiny.fixed_decay_part(heads=4, dim=8, vdim=16, decay=(0.5, 0.8, 0.95, 0.99)), mlp=tiny.moe_mlp(experts=4, top=2, ff=32, groups=2, keep=1)),
               tiny.scan_layer(inner=64, state=8, dt_rank=4, conv=3, mlp=tiny.dense_mlp(48)),
               tiny.channel_decay_layer(heads=2, dim=16, vdim=32, tau=4.0, rank=8, mlp=None)]
     cfg = tiny.make_config(layers, width=64, vocab=70, eps=1e-6, taps=2, loop={"start": 0, "stop": 2, "times": 2})
