@@ -147,3 +147,48 @@ def standard_layers() -> List[dict]:
                        right=fixed_decay_part(heads=2, dim=32, vdim=16, decay=(0.5, 0.99)), mlp=dense_mlp(ff=64)),
             scan_layer(inner=80, state=16, dt_rank=5, conv=2, mlp=moe_mlp(experts=4, top=1, ff=56, groups=1, keep=1)),
             channel_decay_layer(heads=2, dim=40, vdim=24, tau=3.0, rank=16, mlp=moe_mlp(experts=8, top=3, ff=32, groups=4, keep=2))]
+
+
+def random_config(seed: int) -> dict:
+    """A configuration drawn from the design's whole space: 2 .. 5 layers of any kinds in any order, any feed-forward or none,
+    a loop (anywhere, 1 .. 3 passes) or none, 0 .. 5 taps, widths that need not be multiples of 8."""
+    import random
+
+    rnd = random.Random(seed)
+    pick = rnd.choice
+
+    def mlp():
+        kind = pick(["dense", "moe", "moe", None])
+        if kind == "dense":
+            return dense_mlp(ff=pick([24, 40, 66, 128]))
+        if kind == "moe":
+            count = pick([1, 2, 3, 4])
+            per = pick([1, 2, 3])
+            keep = rnd.randint(1, count)
+            return moe_mlp(experts=count * per, top=rnd.randint(1, keep * per), ff=pick([16, 24, 40]), groups=count, keep=keep)
+        return None
+
+    def one():
+        kind = pick(["mamba1", "parallel", "gla"])
+        if kind == "mamba1":
+            return scan_layer(inner=pick([24, 48, 80, 128]), state=pick([1, 4, 7, 16, 24, 40]), dt_rank=pick([1, 3, 8, 12]), conv=pick([1, 2, 4, 6]), mlp=mlp())
+        if kind == "gla":
+            return channel_decay_layer(heads=pick([1, 2, 3, 5]), dim=pick([8, 12, 32, 40]), vdim=pick([8, 20, 32, 64]), tau=pick([1.0, 4.0, 16.0, 30.0]),
+                                       rank=pick([2, 8, 12]), mlp=mlp())
+        G = pick([1, 2, 3, 4])
+        H = G * pick([1, 2, 3, 4])
+        dk = pick([8, 16, 24, 32, 48, 64])
+        Hr = pick([1, 2, 4, 5])
+        left = attention_part(heads=H, kv_heads=G, dim=dk, vdim=pick([8, 16, 32, 48, 80]), scale=pick([0.1, 0.25, dk ** -0.5]),
+                              window=pick([None, 1, 7, 32, 50, 64, 100, 160]), rot_dims=pick([0, 2, dk // 2 // 2 * 2, dk]), rot_base=pick([100.0, 10000.0, 500000.0]))
+        right = fixed_decay_part(heads=Hr, dim=pick([8, 16, 40]), vdim=pick([8, 24, 64]), decay=[rnd.uniform(0.3, 1.0) for _ in range(Hr)])
+        return pair_layer(left=left, right=right, mlp=mlp())
+
+    n = rnd.randint(2, 5)
+    layers = [one() for _ in range(n)]
+    loop = None
+    if rnd.random() < 0.7:
+        a = rnd.randint(0, n - 1)
+        loop = {"start": a, "stop": rnd.randint(a + 1, n), "times": rnd.randint(1, 3)}
+    return make_config(layers, width=pick([24, 36, 40, 64, 100]), vocab=pick([31, 64, 97]), eps=pick([1e-5, 1e-6]), taps=pick([0, 1, 2, 3, 5]),
+                       scale=pick([0.5, 1.0, 3.0]), loop=loop)

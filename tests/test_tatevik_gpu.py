@@ -222,6 +222,38 @@ def test_other_sizes_and_layer_orders(gpu_device, dtype, shape):
     assert close(torch.cat(outs), want, dtype), rel_err(torch.cat(outs), want)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seed", range(16))
+def test_configurations_drawn_at_random(gpu_device, seed, dtype):
+    """Layer kinds, orders, loops, taps and sizes drawn from the design's whole space: a whole prompt, portions with single
+    tokens, and two requests of unequal length in one batch."""
+    cfg = tiny.random_config(seed)
+    tensors = tiny.make_tensors(cfg, seed=100 + seed)
+    lm = build_lm(cfg, tensors, dtype, pages=16)
+    model = ref.TatevikRef(cfg, tensors)
+    a, b = rand_tokens(120, cfg, tensors, 7), rand_tokens(45, cfg, tensors, 8)
+    want_a, want_b = model.forward(a), model.forward(b)
+    with lm.context_manager():
+        seq = lm.open_sequence()
+        whole = lm.step_sequences([(seq, a)])
+        lm.close_sequence(seq)
+        sa, sb = lm.open_sequence(), lm.open_sequence()
+        got_a = [lm.step_sequences([(sa, a[:70])])]
+        out = lm.step_sequences([(sa, a[70:72]), (sb, b[:40])])
+        got_a.append(out[:2])
+        got_b = [out[2:]]
+        for i in range(5):
+            out = lm.step_sequences([(sa, [a[72 + i]]), (sb, [b[40 + i]])])
+            got_a.append(out[:1])
+            got_b.append(out[1:])
+        got_a.append(lm.step_sequences([(sa, a[77:])]))
+        lm.close_sequence(sa)
+        lm.close_sequence(sb)
+    assert close(whole, want_a, dtype), (cfg, rel_err(whole, want_a))
+    assert close(torch.cat(got_a), want_a, dtype), (cfg, rel_err(torch.cat(got_a), want_a))
+    assert close(torch.cat(got_b), want_b, dtype), (cfg, rel_err(torch.cat(got_b), want_b))
+
+
 # ---- mechanisms alone ------------------------------------------------------------------------------------------------------
 class _Step:
     """What a mixer kernel needs to know about a ragged step of sequences that hold `cached` tokens and bring `new` more."""
