@@ -590,10 +590,12 @@ int tgis_selective_scan(const void* x, int64_t ld_x, const void* dt, int64_t ld_
                         int64_t max_q_len, int64_t inner, int N, int dtype, void* stream);
 /* x_out = x_in + s1 * a + s2 * b + v  (each term optional; s1, s2, v [W] fp32; a, b [rows, ld] fp32 or `dtype`), and
  * h = norm(x_out) * w with norm the mean-free layer norm (mean_free) or the RMS norm, eps inside the root; h fp32 (h_f32) or
- * `dtype`; w NULL: no norm.  x_out may alias x_in. */
+ * `dtype`; w NULL: no norm.  x_out may alias x_in.  With a2 (optional) the first term is the average of two normed rows,
+ * pair_coef * (a / rms(a) * wa + a2 / rms(a2) * wa2), instead of a (what tgis_rms_pair_mean makes, without its launch). */
 int tgis_scaled_residual_norm(const float* x_in, float* x_out, const void* a, int64_t ld_a, int a_f32, const float* s1,
                               const void* b, int64_t ld_b, int b_f32, const float* s2, const float* v, const float* w, void* h,
-                              int h_f32, int64_t rows, int64_t W, float eps, int mean_free, int dtype, void* stream);
+                              int h_f32, int64_t rows, int64_t W, float eps, int mean_free, const void* a2, int64_t ld_a2,
+                              int a2_f32, const float* wa, const float* wa2, float pair_coef, int dtype, void* stream);
 /* y = ca * a / rms(a) * wa + cb * b / rms(b) * wb over rows of W channels; a, b fp32 or `dtype`; y fp32. */
 int tgis_rms_pair_mean(const void* a, int64_t ld_a, int a_f32, const float* wa, float ca, const void* b, int64_t ld_b, int b_f32,
                        const float* wb, float cb, float* y, int64_t rows, int64_t W, float eps, int dtype, void* stream);

@@ -538,6 +538,12 @@ def test_feed_forwards_and_row_kernels(gpu_device, dtype, T):
     y = native.rms_pair_mean(a.to(dev), s1.to(dev), 0.5, b2.to(dev), s2.to(dev), 0.5, 1e-5, dtype)
     wy = 0.5 * (ref.rms_unit(a.double(), 1e-5) * s1.double() + ref.rms_unit(b2.double(), 1e-5) * s2.double())
     assert float((y.double().cpu() - wy).abs().max()) < 1e-4
+    # ... and the same average made inside the residual update
+    xo, hn = native.scaled_residual_norm(x.to(dev), a.to(dev), vec.to(dev), None, None, None, w.to(dev), 1e-5, dtype,
+                                         pair=(b2.to(dev), s1.to(dev), s2.to(dev), 0.5))
+    xs = x.double() + vec.double() * wy
+    assert float((xo.double().cpu() - xs).abs().max()) < 1e-4
+    assert float((hn.double().cpu() - ref.layer_norm(xs, w.double(), 1e-5)).abs().max()) < 1e-4
 
 
 # ---- generation through the serving entry points ---------------------------------------------------------------------------

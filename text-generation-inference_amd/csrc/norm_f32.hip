@@ -1,6 +1,7 @@
 // Row kernels over an fp32 residual stream for layers with per-channel scales on their sublayers and a mean-free norm:
 //
-//   tgis_scaled_residual_norm   x <- x + s1 * a + s2 * b + v;   h = norm(x) * w        (norm: layer norm without bias, or RMS)
+//   tgis_scaled_residual_norm   x <- x + s1 * a + s2 * b + v;   h = norm(x) * w        (norm: layer norm without bias, or RMS);
+//                               a may be the average of two normed rows, c (a / rms(a) * wa + a2 / rms(a2) * wa2), made on the way
 //   tgis_rms_pair_mean          y = ca * a / rms(a) * wa + cb * b / rms(b) * wb         (two mixers' results, normed, averaged)
 //   tgis_poly_norm              y = c1 z / rms(z) + c2 z^2 / rms(z^2) + c3 z^3 / rms(z^3) + c0   over a row of feed-forward values
 //
@@ -27,14 +28,28 @@ __global__ __launch_bounds__(256) void scaled_residual_norm_kernel(const float* 
                                                                    int64_t ld_a, int a_f32, const float* __restrict__ s1, const void* b,
                                                                    int64_t ld_b, int b_f32, const float* __restrict__ s2,
                                                                    const float* __restrict__ v, const float* __restrict__ w, void* h,
-                                                                   int h_f32, int W, float eps, int mean_free) {
+                                                                   int h_f32, int W, float eps, int mean_free, const void* a2,
+                                                                   int64_t ld_a2, int a2_f32, const float* __restrict__ wa,
+                                                                   const float* __restrict__ wa2, float pair_coef) {
     extern __shared__ float row[];
     __shared__ float part[4];
     const int64_t t = blockIdx.x;
+    float ra = 1.f, ra2 = 0.f;
+    if (a2) {  // a is a pair of rows, each divided by its root mean square
+        float qa = 0.f, qb = 0.f;
+        for (int c = threadIdx.x; c < W; c += 256) {
+            const float u = ld_as<T>(a, t * ld_a + c, a_f32), u2 = ld_as<T>(a2, t * ld_a2 + c, a2_f32);
+            qa += u * u;
+            qb += u2 * u2;
+        }
+        ra = pair_coef / sqrtf(block_sum(qa, part) / (float)W + eps);
+        ra2 = pair_coef / sqrtf(block_sum(qb, part) / (float)W + eps);
+    }
     float sum = 0.f;
     for (int c = threadIdx.x; c < W; c += 256) {
         float val = x_in ? x_in[t * W + c] : 0.f;
-        if (a) val = fmaf(s1 ? s1[c] : 1.f, ld_as<T>(a, t * ld_a + c, a_f32), val);
+        if (a2) val = fmaf(s1 ? s1[c] : 1.f, ld_as<T>(a, t * ld_a + c, a_f32) * ra * wa[c] + ld_as<T>(a2, t * ld_a2 + c, a2_f32) * ra2 * wa2[c], val);
+        else if (a) val = fmaf(s1 ? s1[c] : 1.f, ld_as<T>(a, t * ld_a + c, a_f32), val);
         if (b) val = fmaf(s2 ? s2[c] : 1.f, ld_as<T>(b, t * ld_b + c, b_f32), val);
         if (v) val += v[c];
         row[c] = val;
@@ -115,7 +130,10 @@ bool dtype_ok(int d) { return d == TGIS_F16 || d == TGIS_BF16 || d == TGIS_F32; 
 
 extern "C" int tgis_scaled_residual_norm(const float* x_in, float* x_out, const void* a, int64_t ld_a, int a_f32, const float* s1,
                                          const void* b, int64_t ld_b, int b_f32, const float* s2, const float* v, const float* w,
-                                         void* h, int h_f32, int64_t rows, int64_t W, float eps, int mean_free, int dtype, void* stream) {
+                                         void* h, int h_f32, int64_t rows, int64_t W, float eps, int mean_free, const void* a2,
+                                         int64_t ld_a2, int a2_f32, const float* wa, const float* wa2, float pair_coef, int dtype,
+                                         void* stream) {
+    TGIS_CHECK_ARG(!a2 || (a && wa && wa2 && ld_a2 >= W), "tgis_scaled_residual_norm: a pair needs both rows and both gains");
     TGIS_CHECK_ARG((x_in || a || b) && (x_out || (w && h)) && (!w || h), "tgis_scaled_residual_norm: nothing to do");
     TGIS_CHECK_ARG(W >= 1 && W * 4 <= 64 * 1024 && (!a || ld_a >= W) && (!b || ld_b >= W) && dtype_ok(dtype),
                    "tgis_scaled_residual_norm: rows of up to 16384 channels (got %ld)", (long)W);
@@ -123,7 +141,7 @@ extern "C" int tgis_scaled_residual_norm(const float* x_in, float* x_out, const 
     hipStream_t st = (hipStream_t)stream;
     TgisTimedScope timed(TGIS_OP_NORM, st);
     BY_DTYPE(dtype, hipLaunchKernelGGL(scaled_residual_norm_kernel<TT>, dim3((unsigned)rows), dim3(256), (size_t)W * 4, st, x_in, x_out, a, ld_a,
-                                       a_f32, s1, b, ld_b, b_f32, s2, v, w, h, h_f32, (int)W, eps, mean_free));
+                                       a_f32, s1, b, ld_b, b_f32, s2, v, w, h, h_f32, (int)W, eps, mean_free, a2, ld_a2, a2_f32, wa, wa2, pair_coef));
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
 }

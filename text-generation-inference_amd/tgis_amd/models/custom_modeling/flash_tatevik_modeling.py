@@ -32,6 +32,8 @@ MIXER_TYPES = ("mamba1", "parallel", "gla")
 PAIR_COEF = 0.5
 # what guards the sum of the chosen experts' scores
 ROUTER_RENORM_EPS = 1e-20
+# rows up to which the pair's average rides in the residual update
+PAIR_FUSED_MAX_ROWS = 256
 
 
 class TatevikConfig:
@@ -183,9 +185,7 @@ class FlashTatevikModel:
         x = x0
         # the normed input of the first run; afterwards a run's residual update also norms for the next one, unless a pass
         # begins there
-        h = self.enter(x, x0, self.layers[0], eps, dt, first=True)
-        if self.layers[0].pass_number is not None:
-            x, h = h
+        x, h = self.enter(x, x0, self.layers[0], eps, dt)
         for r, run in enumerate(self.layers):
             layer = run.layer
             memory = kv.state.shift[run.cache_id]
@@ -195,9 +195,16 @@ class FlashTatevikModel:
             else:
                 h1 = h2 = h
             state = kv.state.state[run.cache_id]
+            pair = None
             if layer.kind == "mamba1":
                 tail = memory[:, layer.canon_floats:layer.canon_floats + layer.mixer_floats] if layer.mixer_floats else None
                 y = layer.mixer.forward(h1, position_ids, kv, state, tail)
+            elif layer.kind == "parallel":
+                # decode-sized steps: the two mixers' rows are normed and averaged by the residual update below (one launch
+                # less); long steps keep the launch of their own (the fused form reads both rows twice)
+                y = layer.mixer.forward(h1, position_ids, kv, run.cache_id, state, defer=h1.shape[0] <= PAIR_FUSED_MAX_ROWS)
+                if isinstance(y, tuple):
+                    y, pair = y
             else:
                 y = layer.mixer.forward(h1, position_ids, kv, run.cache_id, state)
             y_ff = layer.ff(h2) if layer.ff is not None else None
@@ -206,20 +213,19 @@ class FlashTatevikModel:
             gain = (nxt.layer.norm1 if nxt is not None else self.final_norm) if fused else None
             last = nxt is None
             x, h = native.scaled_residual_norm(x, y, layer.ls1, y_ff, layer.ls2, None, gain, eps, dt, x_out=None if x is x0 else x,
-                                               h_f32=not last and cfg.canon_taps > 0)
+                                               h_f32=not last and cfg.canon_taps > 0, pair=pair)
             if kv.residual_trace is not None:
                 kv.residual_trace.append(x.clone())
             if not fused:
                 x, h = self.enter(x, x0, nxt, eps, dt)
         return h  # final-normed, in the serving dtype
 
-    def enter(self, x, x0, run: TatevikRun, eps: float, dt, first: bool = False):
-        """What comes in front of a run: the pass's mix with the embedding and its step vector where a pass begins, then the
-        layer's norm.  Returns the normed input, or (x, normed input) where the stream changed."""
+    def enter(self, x, x0, run: TatevikRun, eps: float, dt):
+        """What comes in front of a run that the run before it did not prepare: where a pass begins, the pass's mix with the
+        embedding and its step vector; then the layer's norm.  Returns (the stream, the normed input)."""
         h_f32 = self.config.canon_taps > 0
         if run.pass_number is None:
-            assert first
-            return native.scaled_residual_norm(x, None, None, None, None, None, run.layer.norm1, eps, dt, h_f32=h_f32, keep_x=False)[1]
+            return x, native.scaled_residual_norm(x, None, None, None, None, None, run.layer.norm1, eps, dt, h_f32=h_f32, keep_x=False)[1]
         both = torch.cat([x, x0], dim=1).to(dt)
         mixed = self.loop_in(both, out_f32=True)
         return native.scaled_residual_norm(mixed, None, None, None, None, self.loop_step[run.pass_number], run.layer.norm1, eps, dt,

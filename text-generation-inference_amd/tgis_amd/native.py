@@ -155,7 +155,7 @@ SIGNATURES = {
     "tgis_selective_scan": (_c_int, [_vp, _c_i64, _vp, _c_i64, _c_int, _vp, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _vp, _vp, _vp, _vp,
                                      _vp, _vp, _vp, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _vp]),
     "tgis_scaled_residual_norm": (_c_int, [_vp, _vp, _vp, _c_i64, _c_int, _vp, _vp, _c_i64, _c_int, _vp, _vp, _vp, _vp, _c_int, _c_i64,
-                                           _c_i64, _c_f, _c_int, _c_int, _vp]),
+                                           _c_i64, _c_f, _c_int, _vp, _c_i64, _c_int, _vp, _vp, _c_f, _c_int, _vp]),
     "tgis_rms_pair_mean": (_c_int, [_vp, _c_i64, _c_int, _vp, _c_f, _vp, _c_i64, _c_int, _vp, _c_f, _vp, _c_i64, _c_i64, _c_f, _c_int, _vp]),
     "tgis_poly_norm": (_c_int, [_vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_f, _c_f, _c_f, _c_f, _c_f, _c_int, _vp]),
     "tgis_moe_route_grouped": (_c_int, [_vp, _c_i64, _vp, _vp, _c_int, _c_int, _c_f, _vp, _vp, _c_i64, _c_i64, _c_int, _c_int, _c_int, _vp]),
@@ -1412,9 +1412,11 @@ def selective_scan(x, dt, dt_bias, bc, b_col0: int, c_col0: int, z, A_log, D, st
 
 
 def scaled_residual_norm(x_in, a, s1, b, s2, v, w, eps: float, act_dtype, x_out=None, h_f32: bool = True, mean_free: bool = True,
-                         keep_x: bool = True):
+                         keep_x: bool = True, pair=None):
     """x_out = x_in + s1 * a + s2 * b + v (every term optional), h = norm(x_out) * w (w None: no norm).  -> (x_out, h); x_out may be
-    x_in; keep_x False: only h is wanted."""
+    x_in; keep_x False: only h is wanted.  pair = (a2, wa, wa2, coef): the first term is coef * (a / rms(a) * wa + a2 / rms(a2) * wa2)."""
+    a2, wa, wa2, coef = pair if pair is not None else (None, None, None, 0.0)
+    assert a2 is None or (a is not None and a2.shape == a.shape and a2.stride(1) == 1 and a2.dtype in (torch.float32, act_dtype))
     ref = x_in if x_in is not None else (a if a is not None else b)
     T, W = ref.shape
     if x_out is None and keep_x:
@@ -1429,7 +1431,8 @@ def scaled_residual_norm(x_in, a, s1, b, s2, v, w, eps: float, act_dtype, x_out=
     _check(load_library().tgis_scaled_residual_norm(
         _ptr(x_in), _ptr(x_out), _ptr(a), a.stride(0) if a is not None else 0, _is_f32(a) if a is not None else 0, _f32(s1, "s1"),
         _ptr(b), b.stride(0) if b is not None else 0, _is_f32(b) if b is not None else 0, _f32(s2, "s2"), _f32(v, "v"), _f32(w, "w"),
-        _ptr(h), int(h_f32 or act_dtype == torch.float32), T, W, float(eps), int(mean_free), dtype_code3(act_dtype), _stream()),
+        _ptr(h), int(h_f32 or act_dtype == torch.float32), T, W, float(eps), int(mean_free), _ptr(a2), a2.stride(0) if a2 is not None else 0,
+        _is_f32(a2) if a2 is not None else 0, _f32(wa, "wa"), _f32(wa2, "wa2"), float(coef), dtype_code3(act_dtype), _stream()),
         "tgis_scaled_residual_norm")
     return x_out, h
 

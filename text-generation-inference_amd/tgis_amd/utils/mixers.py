@@ -696,10 +696,14 @@ class NormedPairMixers:
             self.o.append(lin)
         self.gains = (_f32(weights.get_tensor(left_gain)), _f32(weights.get_tensor(right_gain)))
 
-    def forward(self, h: torch.Tensor, position_ids, step, cache_id: int, state) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, position_ids, step, cache_id: int, state, defer: bool = False):
+        """defer: hand the two projected rows on as (a, (b, gain a, gain b, coef)) for a residual update that norms and
+        averages them on the way (native.scaled_residual_norm(pair=)); else the averaged row."""
         proj = self.stack(h)
         a = self.o[0](self.left.run(proj, self.cols[0], position_ids, step, cache_id, state), out_f32=True)
         b = self.o[1](self.right.run(proj, self.cols[1], position_ids, step, cache_id, state), out_f32=True)
+        if defer:
+            return a, (b, self.gains[0], self.gains[1], self.coef)
         return native.rms_pair_mean(a, self.gains[0], self.coef, b, self.gains[1], self.coef, self.eps, h.dtype)
 
 
