@@ -487,6 +487,9 @@ constexpr int P_ROW = 40;     // T elements per query row of a weight tile (80 b
 
 // the value of the lane N places further on in its row of 16 lanes (a data-parallel-primitive move: no trip through LDS); four of
 // them with N = 8, 4, 2, 1 leave a row's sum or maximum in all of its lanes
+// e^x by the hardware's base-two exponential (fp32, a few units in the last place): this form serves two-byte models, whose
+// weights are rounded to two bytes for the last product anyway
+__device__ __forceinline__ float exp_hw(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
 template <int N> __device__ __forceinline__ float row_ror(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x120 + N, 0xF, 0xF, true));
 }
@@ -600,13 +603,13 @@ __global__ __launch_bounds__(512) void attn_mixed_mfma_kernel(MixArgs a) {
                     mx = fmaxf(mx, row_ror<2>(mx));
                     mx = fmaxf(mx, row_ror<1>(mx));
                     const float m_new = fmaxf(mrun[i][u], mx);
-                    const float pa = va ? expf(xa - m_new) : 0.f, pb2 = vb ? expf(xb - m_new) : 0.f;
+                    const float pa = va ? exp_hw(xa - m_new) : 0.f, pb2 = vb ? exp_hw(xb - m_new) : 0.f;
                     float ps = pa + pb2;
                     ps += row_ror<8>(ps);
                     ps += row_ror<4>(ps);
                     ps += row_ror<2>(ps);
                     ps += row_ror<1>(ps);
-                    const float f = m_new == -INFINITY ? 1.f : expf(mrun[i][u] - m_new);
+                    const float f = m_new == -INFINITY ? 1.f : exp_hw(mrun[i][u] - m_new);
                     lrun[i][u] = lrun[i][u] * f + ps;
                     mrun[i][u] = m_new;
                     if (f != 1.f) {

@@ -23,7 +23,7 @@ template <typename T> __device__ __forceinline__ float ld_as(const void* p, int6
     return f32 ? reinterpret_cast<const float*>(p)[i] : (float)reinterpret_cast<const T*>(p)[i];
 }
 
-template <typename T>
+template <typename T, bool PAIR>
 __global__ __launch_bounds__(256) void scaled_residual_norm_kernel(const float* x_in, float* x_out, const void* a,
                                                                    int64_t ld_a, int a_f32, const float* __restrict__ s1, const void* b,
                                                                    int64_t ld_b, int b_f32, const float* __restrict__ s2,
@@ -35,7 +35,7 @@ __global__ __launch_bounds__(256) void scaled_residual_norm_kernel(const float* 
     __shared__ float part[4];
     const int64_t t = blockIdx.x;
     float ra = 1.f, ra2 = 0.f;
-    if (a2) {  // a is a pair of rows, each divided by its root mean square
+    if (PAIR) {  // a is a pair of rows, each divided by its root mean square
         float qa = 0.f, qb = 0.f;
         for (int c = threadIdx.x; c < W; c += 256) {
             const float u = ld_as<T>(a, t * ld_a + c, a_f32), u2 = ld_as<T>(a2, t * ld_a2 + c, a2_f32);
@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) void scaled_residual_norm_kernel(const float* 
     float sum = 0.f;
     for (int c = threadIdx.x; c < W; c += 256) {
         float val = x_in ? x_in[t * W + c] : 0.f;
-        if (a2) val = fmaf(s1 ? s1[c] : 1.f, ld_as<T>(a, t * ld_a + c, a_f32) * ra * wa[c] + ld_as<T>(a2, t * ld_a2 + c, a2_f32) * ra2 * wa2[c], val);
+        if (PAIR) val = fmaf(s1 ? s1[c] : 1.f, ld_as<T>(a, t * ld_a + c, a_f32) * ra * wa[c] + ld_as<T>(a2, t * ld_a2 + c, a2_f32) * ra2 * wa2[c], val);
         else if (a) val = fmaf(s1 ? s1[c] : 1.f, ld_as<T>(a, t * ld_a + c, a_f32), val);
         if (b) val = fmaf(s2 ? s2[c] : 1.f, ld_as<T>(b, t * ld_b + c, b_f32), val);
         if (v) val += v[c];
@@ -140,8 +140,14 @@ extern "C" int tgis_scaled_residual_norm(const float* x_in, float* x_out, const 
     if (rows == 0) return TGIS_OK;
     hipStream_t st = (hipStream_t)stream;
     TgisTimedScope timed(TGIS_OP_NORM, st);
-    BY_DTYPE(dtype, hipLaunchKernelGGL(scaled_residual_norm_kernel<TT>, dim3((unsigned)rows), dim3(256), (size_t)W * 4, st, x_in, x_out, a, ld_a,
-                                       a_f32, s1, b, ld_b, b_f32, s2, v, w, h, h_f32, (int)W, eps, mean_free, a2, ld_a2, a2_f32, wa, wa2, pair_coef));
+    if (a2)
+        BY_DTYPE(dtype, hipLaunchKernelGGL((scaled_residual_norm_kernel<TT, true>), dim3((unsigned)rows), dim3(256), (size_t)W * 4, st, x_in, x_out, a,
+                                           ld_a, a_f32, s1, b, ld_b, b_f32, s2, v, w, h, h_f32, (int)W, eps, mean_free, a2, ld_a2, a2_f32, wa, wa2,
+                                           pair_coef));
+    else
+        BY_DTYPE(dtype, hipLaunchKernelGGL((scaled_residual_norm_kernel<TT, false>), dim3((unsigned)rows), dim3(256), (size_t)W * 4, st, x_in, x_out, a,
+                                           ld_a, a_f32, s1, b, ld_b, b_f32, s2, v, w, h, h_f32, (int)W, eps, mean_free, a2, ld_a2, a2_f32, wa, wa2,
+                                           pair_coef));
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
 }
